@@ -1,0 +1,497 @@
+// Host side of libgalvatron_dp_hip.so: the C ABI declared in include/galvatron_dp_hip.h.
+//
+// A plan owns one device allocation, one stream and the events used for timing; nothing is shared
+// between plans, so calls from different threads never touch common mutable state.
+#include "../../include/galvatron_dp_hip.h"
+#include "gdp_kernels.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string &msg)
+{
+    g_err = msg;
+    return code;
+}
+
+int fail_hip(hipError_t e, const char *what)
+{
+    // a failed allocation is reported as such; everything else as a runtime error
+    const int code = (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) ? GDP_E_NOMEM : GDP_E_HIP;
+    return fail(code, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define GDP_HIP(call)                                    \
+    do {                                                 \
+        hipError_t e_ = (call);                          \
+        if (e_ != hipSuccess) return fail_hip(e_, #call); \
+    } while (0)
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct HostInst {
+    int orig;  // index in the caller's arrays
+    int L, V, S, SP, P, ntile, n_key, n_inter;
+    int64_t ld, ldm;
+    uint32_t flags;
+    int key_begin;  // first entry in the key table
+    int res_begin;  // first element in the result array
+    // byte offsets inside the device allocation
+    size_t off_H0, off_H1, off_M, off_inter, off_intra, off_index, off_roff, off_mem;
+};
+
+struct Group {  // instances with the same S, sorted by L descending
+    int first, count, SP, S, max_L, max_ntile;
+    int64_t max_ld;
+    std::vector<int> active;  // active[l] = number of instances with L > l
+};
+
+}  // namespace
+
+struct gdp_plan {
+    int n = 0;
+    int device = 0;
+    std::vector<HostInst> inst;  // sorted order
+    std::vector<Group> groups;
+    char *dbase = nullptr;
+    size_t dbytes = 0;
+    size_t off_insts = 0, off_keys = 0, off_out = 0, off_res = 0;
+    int n_key_total = 0;
+    size_t n_res_total = 0;
+    int max_L = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    std::vector<hipEvent_t> ev_relax;  // pairs
+    std::vector<GdpDevOut> h_out;
+    std::vector<int32_t> h_res;
+    double relaxations = 0, relax_bytes = 0;
+    bool ran = false;
+};
+
+namespace {
+
+int validate(const gdp_problem *p, int i)
+{
+    char buf[160];
+    auto bad = [&](int code, const char *why) {
+        snprintf(buf, sizeof buf, "instance %d: %s", i, why);
+        return fail(code, buf);
+    };
+    if (!p) return bad(GDP_E_BADARG, "null problem");
+    if (p->L < 1 || p->V < 1 || p->S < 1) return bad(GDP_E_BADARG, "L, V and S must be >= 1");
+    if (p->S > GDP_MAX_S) return bad(GDP_E_BADARG, "S exceeds GDP_MAX_S");
+    if (!p->mem || !p->intra || !p->inter) return bad(GDP_E_BADARG, "null input array");
+    if (p->n_key < 0 || (p->n_key > 0 && (!p->other_mem || !p->other_time)))
+        return bad(GDP_E_BADARG, "bad key arrays");
+    const int T = p->inter_index ? p->n_inter : p->L;
+    if (T < 1) return bad(GDP_E_BADARG, "n_inter must be >= 1");
+    const size_t LS = (size_t)p->L * p->S;
+    for (size_t k = 0; k < LS; ++k) {
+        if (p->mem[k] < 0) return bad(GDP_E_BADARG, "negative mem entry");
+        if (p->mem[k] == 0)
+            return bad(GDP_E_UNSUPPORTED, "mem entry equal to 0 (in-place update reads its own row)");
+    }
+    if (p->inter_index)
+        for (int l = 0; l < p->L; ++l)
+            if (p->inter_index[l] < 0 || p->inter_index[l] >= T) return bad(GDP_E_BADARG, "inter_index out of range");
+    // NaN and -inf make the reference's result depend on evaluation order; reject them, and
+    // make sure no partial sum can overflow to an infinity of either sign.
+    double bound = 0;
+    for (int l = 0; l < p->L; ++l) {
+        double m = 0;
+        for (int s = 0; s < p->S; ++s) {
+            const double x = p->intra[(size_t)l * p->S + s];
+            if (x != x || x == -INFINITY) return bad(GDP_E_NONFINITE, "NaN or -inf in intra");
+            if (x != INFINITY) m = std::max(m, std::fabs(x));
+        }
+        bound += m;
+    }
+    std::vector<double> tmax((size_t)T, 0.0);
+    const size_t SS = (size_t)p->S * p->S;
+    for (int t = 0; t < T; ++t) {
+        double m = 0;
+        const double *q = p->inter + (size_t)t * SS;
+        for (size_t k = 0; k < SS; ++k) {
+            const double x = q[k];
+            if (x != x || x == -INFINITY) return bad(GDP_E_NONFINITE, "NaN or -inf in inter");
+            if (x != INFINITY) m = std::max(m, std::fabs(x));
+        }
+        tmax[t] = m;
+    }
+    for (int l = 0; l < p->L; ++l) bound += tmax[p->inter_index ? p->inter_index[l] : l];
+    for (int k = 0; k < p->n_key; ++k) {
+        const double x = p->other_time[k];
+        if (x != x || x == -INFINITY) return bad(GDP_E_NONFINITE, "NaN or -inf in other_time");
+    }
+    if (!(bound < 1e300)) return bad(GDP_E_NONFINITE, "cost magnitudes could overflow binary64");
+    return GDP_OK;
+}
+
+void destroy(gdp_plan *pl)
+{
+    if (!pl) return;
+    if (pl->dbase) (void)hipFree(pl->dbase);
+    for (hipEvent_t e : pl->ev_relax) (void)hipEventDestroy(e);
+    if (pl->ev_begin) (void)hipEventDestroy(pl->ev_begin);
+    if (pl->ev_end) (void)hipEventDestroy(pl->ev_end);
+    if (pl->stream) (void)hipStreamDestroy(pl->stream);
+    delete pl;
+}
+
+int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
+{
+    pl->n = n;
+    GDP_HIP(hipGetDevice(&pl->device));
+    // ---- shapes -------------------------------------------------------------------------------
+    std::vector<HostInst> inst((size_t)n);
+    for (int i = 0; i < n; ++i) {
+        const gdp_problem *q = p[i];
+        HostInst &h = inst[(size_t)i];
+        h.orig = i;
+        h.L = q->L; h.V = q->V; h.S = q->S;
+        h.SP = (int)align_up((size_t)q->S, GDP_TS);
+        h.n_key = q->n_key;
+        h.n_inter = q->inter_index ? q->n_inter : q->L;
+        h.flags = q->flags;
+        int maxm = 0;
+        for (size_t k = 0; k < (size_t)q->L * q->S; ++k)
+            if (q->mem[k] < q->V) maxm = std::max(maxm, q->mem[k]);
+        h.P = (int)align_up((size_t)std::max(maxm, 1), 64);
+        h.ntile = (q->V + GDP_TILE_ROWS - 1) / GDP_TILE_ROWS;
+        h.ldm = (int64_t)h.ntile * GDP_TILE_ROWS;
+        h.ld = h.P + h.ldm;
+    }
+    // group by S, then by L descending (stable, so equal shapes keep the caller's order)
+    std::stable_sort(inst.begin(), inst.end(), [](const HostInst &a, const HostInst &b) {
+        if (a.S != b.S) return a.S < b.S;
+        return a.L > b.L;
+    });
+    for (int i = 0; i < n;) {
+        Group g;
+        g.first = i; g.S = inst[(size_t)i].S; g.SP = inst[(size_t)i].SP;
+        g.max_L = 0; g.max_ntile = 0; g.max_ld = 0;
+        int j = i;
+        while (j < n && inst[(size_t)j].S == g.S) {
+            g.max_L = std::max(g.max_L, inst[(size_t)j].L);
+            g.max_ntile = std::max(g.max_ntile, inst[(size_t)j].ntile);
+            g.max_ld = std::max(g.max_ld, inst[(size_t)j].ld);
+            ++j;
+        }
+        g.count = j - i;
+        g.active.assign((size_t)g.max_L, 0);
+        for (int k = i; k < j; ++k)
+            for (int l = 0; l < inst[(size_t)k].L; ++l) g.active[(size_t)l]++;
+        pl->max_L = std::max(pl->max_L, g.max_L);
+        pl->groups.push_back(g);
+        i = j;
+    }
+    // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t o = off;
+        off = align_up(off + bytes, 256);
+        return o;
+    };
+    int nk = 0;
+    size_t nres = 0;
+    for (auto &h : inst) {
+        h.key_begin = nk; nk += h.n_key;
+        h.res_begin = (int)nres; nres += (size_t)h.n_key * h.L;
+    }
+    pl->n_key_total = nk;
+    pl->n_res_total = nres;
+    pl->off_insts = take(sizeof(GdpDevInst) * (size_t)n);
+    pl->off_keys = take(sizeof(GdpDevKey) * (size_t)std::max(nk, 1));
+    for (auto &h : inst) {
+        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.S + 1) * h.SP);
+        h.off_intra = take(sizeof(double) * (size_t)h.L * h.SP);
+        h.off_index = take(sizeof(int32_t) * (size_t)h.L);
+        h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.S + 1));
+        h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
+    }
+    const size_t small_bytes = off;
+    pl->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(nk, 1));
+    pl->off_res = take(sizeof(int32_t) * std::max<size_t>(nres, 1));
+    for (auto &h : inst) {
+        h.off_H0 = take(sizeof(double) * (size_t)(h.S + 1) * (size_t)h.ld);
+        h.off_H1 = take(sizeof(double) * (size_t)(h.S + 1) * (size_t)h.ld);
+        h.off_M = take((size_t)h.L * h.S * (size_t)h.ldm);
+    }
+    pl->dbytes = off;
+    {
+        hipError_t e = hipMalloc((void **)&pl->dbase, pl->dbytes);
+        if (e != hipSuccess) {
+            char buf[128];
+            snprintf(buf, sizeof buf, "hipMalloc of %zu bytes", pl->dbytes);
+            return fail_hip(e, buf);
+        }
+    }
+    // ---- build the small region on the host ------------------------------------------------------
+    std::vector<char> stage;
+    try {
+        stage.assign(small_bytes, 0);
+    } catch (const std::bad_alloc &) {
+        return fail(GDP_E_NOMEM, "host staging allocation failed");
+    }
+    GdpDevInst *di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
+    GdpDevKey *dk = reinterpret_cast<GdpDevKey *>(stage.data() + pl->off_keys);
+    for (int i = 0; i < n; ++i) {
+        const HostInst &h = inst[(size_t)i];
+        const gdp_problem *q = p[h.orig];
+        GdpDevInst &d = di[i];
+        d.H[0] = reinterpret_cast<double *>(pl->dbase + h.off_H0);
+        d.H[1] = reinterpret_cast<double *>(pl->dbase + h.off_H1);
+        d.M = reinterpret_cast<uint8_t *>(pl->dbase + h.off_M);
+        d.inter = reinterpret_cast<const double *>(pl->dbase + h.off_inter);
+        d.intra = reinterpret_cast<const double *>(pl->dbase + h.off_intra);
+        d.inter_index = reinterpret_cast<const int32_t *>(pl->dbase + h.off_index);
+        d.roff = reinterpret_cast<const int64_t *>(pl->dbase + h.off_roff);
+        d.mem = reinterpret_cast<const int32_t *>(pl->dbase + h.off_mem);
+        d.ld = h.ld; d.ldm = h.ldm;
+        d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.P = h.P; d.ntile = h.ntile;
+        d.pad0 = d.pad1 = 0;
+        // inter: [T][S+1][SP], zero padded
+        double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
+        for (int t = 0; t < h.n_inter; ++t)
+            for (int a = 0; a < h.S; ++a)
+                memcpy(it + ((size_t)t * (h.S + 1) + a) * h.SP, q->inter + ((size_t)t * h.S + a) * h.S,
+                       sizeof(double) * (size_t)h.S);
+        double *ia = reinterpret_cast<double *>(stage.data() + h.off_intra);
+        for (int l = 0; l < h.L; ++l)
+            memcpy(ia + (size_t)l * h.SP, q->intra + (size_t)l * h.S, sizeof(double) * (size_t)h.S);
+        int32_t *ix = reinterpret_cast<int32_t *>(stage.data() + h.off_index);
+        for (int l = 0; l < h.L; ++l) ix[l] = q->inter_index ? q->inter_index[l] : l;
+        memcpy(stage.data() + h.off_mem, q->mem, sizeof(int32_t) * (size_t)h.L * h.S);
+        // roff[l][s']: where row 0 of "f after layer l-1, strategy s'" sits in a cost buffer
+        int64_t *ro = reinterpret_cast<int64_t *>(stage.data() + h.off_roff);
+        const int64_t inf_row = (int64_t)h.S * h.ld + h.P;
+        for (int l = 0; l <= h.L; ++l) {
+            int64_t *row = ro + (size_t)l * (h.S + 1);
+            for (int s = 0; s < h.S; ++s) {
+                if (l == 0) {
+                    row[s] = (int64_t)s * h.ld + h.P;  // zeros: the caller's initial f
+                } else {
+                    const int m = q->mem[(size_t)(l - 1) * h.S + s];
+                    row[s] = (m >= h.V) ? inf_row : (int64_t)s * h.ld + h.P - m;
+                }
+            }
+            row[h.S] = row[0];  // target of the last prefetch
+        }
+        for (int k = 0; k < h.n_key; ++k) {
+            GdpDevKey &key = dk[h.key_begin + k];
+            key.other_mem = q->other_mem[k];
+            key.other_time = q->other_time[k];
+            key.inst = i;
+            key.res_off = h.res_begin + k * h.L;
+        }
+        pl->relaxations += (double)h.L * h.V * (double)h.S * h.S;
+        pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + 1);
+    }
+    GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));
+    GDP_HIP(hipEventCreate(&pl->ev_begin));
+    GDP_HIP(hipEventCreate(&pl->ev_end));
+    GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
+    GDP_HIP(hipStreamSynchronize(pl->stream));
+    pl->inst.swap(inst);
+    pl->h_out.resize((size_t)std::max(nk, 1));
+    pl->h_res.resize(std::max<size_t>(nres, 1));
+    return GDP_OK;
+}
+
+int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
+{
+    GDP_HIP(hipSetDevice(pl->device));
+    const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
+    const GdpDevKey *d_keys = reinterpret_cast<const GdpDevKey *>(pl->dbase + pl->off_keys);
+    GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
+    int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
+    size_t launches = 0;
+    for (const Group &g : pl->groups) launches += (size_t)g.max_L;
+    if (mode >= 2)
+        while (pl->ev_relax.size() < 2 * launches) {
+            hipEvent_t e;
+            GDP_HIP(hipEventCreate(&e));
+            pl->ev_relax.push_back(e);
+        }
+    if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_begin, pl->stream));
+    for (const Group &g : pl->groups)
+        GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, pl->stream));
+    size_t li = 0;
+    for (int l = 0; l < pl->max_L; ++l)
+        for (const Group &g : pl->groups) {
+            if (l >= g.max_L) continue;
+            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
+            GDP_HIP(gdp_launch_relax(d_insts + g.first, g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
+            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
+            ++li;
+        }
+    GDP_HIP(gdp_launch_epilogue(d_insts, d_keys, pl->n_key_total, d_out, d_res, pl->stream));
+    if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
+    GDP_HIP(hipStreamSynchronize(pl->stream));
+    pl->ran = true;
+    if (t) {
+        memset(t, 0, sizeof *t);
+        t->relaxations = pl->relaxations;
+        t->relax_bytes = pl->relax_bytes;
+        t->relax_launches = (int32_t)launches;
+        if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));
+        if (mode >= 2) {
+            float sum = 0;
+            for (size_t k = 0; k < launches; ++k) {
+                float ms = 0;
+                GDP_HIP(hipEventElapsedTime(&ms, pl->ev_relax[2 * k], pl->ev_relax[2 * k + 1]));
+                sum += ms;
+            }
+            t->relax_ms = sum;
+        }
+    }
+    return GDP_OK;
+}
+
+int fetch(gdp_plan *pl, gdp_result *const *r)
+{
+    if (!pl->ran) return fail(GDP_E_BADARG, "gdp_plan_fetch before gdp_plan_run");
+    GDP_HIP(hipSetDevice(pl->device));
+    if (pl->n_key_total > 0) {
+        GDP_HIP(hipMemcpyAsync(pl->h_out.data(), pl->dbase + pl->off_out, sizeof(GdpDevOut) * (size_t)pl->n_key_total,
+                               hipMemcpyDeviceToHost, pl->stream));
+        GDP_HIP(hipMemcpyAsync(pl->h_res.data(), pl->dbase + pl->off_res, sizeof(int32_t) * pl->n_res_total,
+                               hipMemcpyDeviceToHost, pl->stream));
+        GDP_HIP(hipStreamSynchronize(pl->stream));
+    }
+    const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
+    for (int i = 0; i < pl->n; ++i) {
+        const HostInst &h = pl->inst[(size_t)i];
+        gdp_result *out = r[h.orig];
+        if (!out) return fail(GDP_E_BADARG, "null result");
+        if (h.n_key > 0 && (!out->total || !out->remaining || !out->res)) return fail(GDP_E_BADARG, "null result array");
+        for (int k = 0; k < h.n_key; ++k) {
+            const GdpDevOut &o = pl->h_out[(size_t)(h.key_begin + k)];
+            out->total[k] = o.total;
+            out->remaining[k] = o.remaining;
+            if (o.feasible)
+                memcpy(out->res + (size_t)k * h.L, pl->h_res.data() + h.res_begin + (size_t)k * h.L,
+                       sizeof(int32_t) * (size_t)h.L);
+        }
+        if ((h.flags & GDP_EXPORT_F) && out->f_out) {
+            double *tmp = nullptr;
+            const size_t bytes = sizeof(double) * (size_t)h.V * h.S;
+            GDP_HIP(hipMalloc((void **)&tmp, bytes));
+            hipError_t e = gdp_launch_export_f(d_insts + i, tmp, h.V, h.S, pl->stream);
+            if (e == hipSuccess) e = hipMemcpyAsync(out->f_out, tmp, bytes, hipMemcpyDeviceToHost, pl->stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(pl->stream);
+            (void)hipFree(tmp);
+            if (e != hipSuccess) return fail_hip(e, "export f");
+        }
+        if ((h.flags & GDP_EXPORT_MARK) && out->mark_out) {
+            int32_t *tmp = nullptr;
+            const size_t bytes = sizeof(int32_t) * (size_t)h.V * h.S;
+            GDP_HIP(hipMalloc((void **)&tmp, bytes));
+            hipError_t e = hipSuccess;
+            for (int l = 0; l < h.L && e == hipSuccess; ++l) {
+                e = gdp_launch_export_mark(d_insts + i, l, tmp, h.V, h.S, pl->stream);
+                if (e == hipSuccess)
+                    e = hipMemcpyAsync(out->mark_out + (size_t)l * h.V * h.S, tmp, bytes, hipMemcpyDeviceToHost,
+                                       pl->stream);
+                if (e == hipSuccess) e = hipStreamSynchronize(pl->stream);
+            }
+            (void)hipFree(tmp);
+            if (e != hipSuccess) return fail_hip(e, "export mark");
+        }
+    }
+    return GDP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
+{
+    g_err.clear();
+    if (!out) return fail(GDP_E_BADARG, "null plan pointer");
+    *out = nullptr;
+    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
+    if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
+    for (int i = 0; i < n; ++i) {
+        int rc = validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+    }
+    gdp_plan *pl = new (std::nothrow) gdp_plan();
+    if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
+    int rc;
+    try {
+        rc = create(n, p, pl);
+    } catch (const std::bad_alloc &) {
+        rc = fail(GDP_E_NOMEM, "host allocation failed");
+    }
+    if (rc != GDP_OK) {
+        destroy(pl);
+        return rc;
+    }
+    *out = pl;
+    return GDP_OK;
+}
+
+int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing)
+{
+    g_err.clear();
+    if (!plan) return fail(GDP_E_BADARG, "null plan");
+    return run(plan, timing ? timing_mode : 0, timing);
+}
+
+int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r)
+{
+    g_err.clear();
+    if (!plan || !r) return fail(GDP_E_BADARG, "null plan or results");
+    return fetch(plan, r);
+}
+
+void gdp_plan_destroy(gdp_plan *plan) { destroy(plan); }
+
+int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
+{
+    if (!r) return fail(GDP_E_BADARG, "null results");
+    gdp_plan *pl = nullptr;
+    int rc = gdp_plan_create(n, p, &pl);
+    if (rc != GDP_OK) return rc;
+    rc = run(pl, 0, nullptr);
+    if (rc == GDP_OK) rc = fetch(pl, r);
+    destroy(pl);
+    return rc;
+}
+
+int gdp_solve(const gdp_problem *p, gdp_result *r)
+{
+    const gdp_problem *pp[1] = {p};
+    gdp_result *rr[1] = {r};
+    return gdp_solve_batch(1, pp, rr);
+}
+
+const char *gdp_last_error(void) { return g_err.c_str(); }
+
+int gdp_version(void) { return GDP_VERSION; }
+
+int gdp_device_info(char *buf, size_t len)
+{
+    g_err.clear();
+    if (!buf || len == 0) return fail(GDP_E_BADARG, "null buffer");
+    int dev = 0;
+    GDP_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    GDP_HIP(hipGetDeviceProperties(&prop, dev));
+    snprintf(buf, len, "%s;%s;%d;%zu", prop.name, prop.gcnArchName, prop.multiProcessorCount,
+             (size_t)prop.totalGlobalMem);
+    return GDP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,211 @@
+"""ctypes binding of libgalvatron_dp_hip.so (the C ABI in include/galvatron_dp_hip.h).
+
+There is no CPU fallback: if the HIP library has not been built, or no HIP device is usable,
+every compute call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Sequence
+
+import numpy as np
+
+PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(PKG, "lib", "libgalvatron_dp_hip.so")
+
+GDP_OK = 0
+GDP_E_BADARG = -1
+GDP_E_UNSUPPORTED = -2
+GDP_E_NONFINITE = -3
+GDP_E_NOMEM = -4
+GDP_E_HIP = -5
+GDP_EXPORT_F = 1
+GDP_EXPORT_MARK = 2
+GDP_MAX_S = 256
+
+EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
+                    "gdp_plan_destroy", "gdp_last_error", "gdp_version", "gdp_device_info")
+
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_f64p = ctypes.POINTER(ctypes.c_double)
+
+
+class UnsupportedInputError(ValueError):
+    """Input outside what the device recurrence covers (a memory cost of 0)."""
+
+
+class gdp_problem(ctypes.Structure):
+    _fields_ = [("L", ctypes.c_int32), ("V", ctypes.c_int32), ("S", ctypes.c_int32),
+                ("mem", _i32p), ("intra", _f64p), ("inter", _f64p), ("inter_index", _i32p),
+                ("n_inter", ctypes.c_int32), ("n_key", ctypes.c_int32),
+                ("other_mem", _i64p), ("other_time", _f64p), ("flags", ctypes.c_uint32)]
+
+
+class gdp_result(ctypes.Structure):
+    _fields_ = [("total", _f64p), ("remaining", _i32p), ("res", _i32p), ("f_out", _f64p), ("mark_out", _i32p)]
+
+
+class gdp_timing(ctypes.Structure):
+    _fields_ = [("total_ms", ctypes.c_float), ("relax_ms", ctypes.c_float), ("relax_launches", ctypes.c_int32),
+                ("reserved", ctypes.c_int32), ("relaxations", ctypes.c_double), ("relax_bytes", ctypes.c_double)]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python __graft_entry__.py` "
+                               "(galvatron_dp._build.build()); there is no CPU fallback")
+        L = ctypes.CDLL(LIB_PATH)
+        pp = ctypes.POINTER(ctypes.POINTER(gdp_problem))
+        rp = ctypes.POINTER(ctypes.POINTER(gdp_result))
+        L.gdp_solve.argtypes = [ctypes.POINTER(gdp_problem), ctypes.POINTER(gdp_result)]
+        L.gdp_solve.restype = ctypes.c_int
+        L.gdp_solve_batch.argtypes = [ctypes.c_int32, pp, rp]
+        L.gdp_solve_batch.restype = ctypes.c_int
+        L.gdp_plan_create.argtypes = [ctypes.c_int32, pp, ctypes.POINTER(ctypes.c_void_p)]
+        L.gdp_plan_create.restype = ctypes.c_int
+        L.gdp_plan_run.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(gdp_timing)]
+        L.gdp_plan_run.restype = ctypes.c_int
+        L.gdp_plan_fetch.argtypes = [ctypes.c_void_p, rp]
+        L.gdp_plan_fetch.restype = ctypes.c_int
+        L.gdp_plan_destroy.argtypes = [ctypes.c_void_p]
+        L.gdp_plan_destroy.restype = None
+        L.gdp_last_error.argtypes = []
+        L.gdp_last_error.restype = ctypes.c_char_p
+        L.gdp_version.argtypes = []
+        L.gdp_version.restype = ctypes.c_int
+        L.gdp_device_info.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+        L.gdp_device_info.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc == GDP_OK:
+        return
+    msg = lib().gdp_last_error().decode("utf-8", "replace")
+    if rc == GDP_E_UNSUPPORTED:
+        raise UnsupportedInputError(msg)
+    if rc in (GDP_E_BADARG, GDP_E_NONFINITE):
+        raise ValueError(msg)
+    if rc == GDP_E_NOMEM:
+        raise MemoryError(msg)
+    raise RuntimeError(f"galvatron_dp_hip error {rc}: {msg}")
+
+
+def device_info() -> str:
+    buf = ctypes.create_string_buffer(256)
+    _check(lib().gdp_device_info(buf, 256))
+    return buf.value.decode()
+
+
+class Problem:
+    """One DP instance (the arguments of one reference plugin call) with host arrays in the
+    dtypes/layouts the C ABI wants, plus the output arrays it will fill."""
+
+    def __init__(self, mem, intra, inter, V: int, other_mem: Sequence[int], other_time: Sequence[float], *,
+                 inter_index=None, export_f: bool = False, export_mark: bool = False):
+        self.mem = np.ascontiguousarray(mem, dtype=np.int32)
+        if self.mem.ndim != 2:
+            raise ValueError("mem must be [L,S]")
+        self.L, self.S = (int(x) for x in self.mem.shape)
+        self.V = int(V)
+        self.intra = np.ascontiguousarray(intra, dtype=np.float64)
+        self.inter = np.ascontiguousarray(inter, dtype=np.float64)
+        if self.intra.shape != (self.L, self.S):
+            raise ValueError("intra must be [L,S]")
+        if self.inter.ndim != 3 or self.inter.shape[1:] != (self.S, self.S):
+            raise ValueError("inter must be [T,S,S]")
+        if inter_index is None:
+            if self.inter.shape[0] != self.L:
+                raise ValueError("inter must be [L,S,S] when inter_index is not given")
+            self.inter_index = None
+        else:
+            self.inter_index = np.ascontiguousarray(inter_index, dtype=np.int32)
+            if self.inter_index.shape != (self.L,):
+                raise ValueError("inter_index must be [L]")
+        self.other_mem = np.ascontiguousarray(other_mem, dtype=np.int64).reshape(-1)
+        self.other_time = np.ascontiguousarray(other_time, dtype=np.float64).reshape(-1)
+        if self.other_mem.shape != self.other_time.shape:
+            raise ValueError("other_mem and other_time must have one entry per key")
+        self.n_key = int(self.other_mem.shape[0])
+        self.flags = (GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0)
+        if self.V < 1 or self.L < 1 or self.S < 1:
+            raise ValueError("L, V and S must be >= 1")
+        # outputs
+        self.total = np.full(self.n_key, np.inf, dtype=np.float64)
+        self.remaining = np.full(self.n_key, -1, dtype=np.int32)
+        self.res = np.full((self.n_key, self.L), -1, dtype=np.int32)
+        self.f_out = np.empty((self.V, self.S), dtype=np.float64) if export_f else None
+        self.mark_out = np.empty((self.L, self.V, self.S), dtype=np.int32) if export_mark else None
+        self._c_problem = gdp_problem(
+            self.L, self.V, self.S, self.mem.ctypes.data_as(_i32p), self.intra.ctypes.data_as(_f64p),
+            self.inter.ctypes.data_as(_f64p),
+            None if self.inter_index is None else self.inter_index.ctypes.data_as(_i32p),
+            int(self.inter.shape[0]), self.n_key, self.other_mem.ctypes.data_as(_i64p),
+            self.other_time.ctypes.data_as(_f64p), self.flags)
+        self._c_result = gdp_result(
+            self.total.ctypes.data_as(_f64p), self.remaining.ctypes.data_as(_i32p), self.res.ctypes.data_as(_i32p),
+            None if self.f_out is None else self.f_out.ctypes.data_as(_f64p),
+            None if self.mark_out is None else self.mark_out.ctypes.data_as(_i32p))
+
+    @property
+    def relaxations(self) -> int:
+        return self.L * self.V * self.S * self.S
+
+
+def _arrays(problems: Sequence[Problem]):
+    n = len(problems)
+    P = (ctypes.POINTER(gdp_problem) * n)(*[ctypes.pointer(p._c_problem) for p in problems])
+    R = (ctypes.POINTER(gdp_result) * n)(*[ctypes.pointer(p._c_result) for p in problems])
+    return P, R
+
+
+def solve_batch(problems: Sequence[Problem]) -> None:
+    """gdp_solve_batch: fills ``total``/``remaining``/``res`` (and exports) of every problem."""
+    if not problems:
+        return
+    P, R = _arrays(problems)
+    _check(lib().gdp_solve_batch(len(problems), P, R))
+
+
+class Plan:
+    """gdp_plan_*: inputs resident on the device, the device part runnable repeatedly."""
+
+    def __init__(self, problems: Sequence[Problem]):
+        self.problems = list(problems)
+        self._P, self._R = _arrays(self.problems)
+        h = ctypes.c_void_p()
+        _check(lib().gdp_plan_create(len(self.problems), self._P, ctypes.byref(h)))
+        self._h = h
+
+    def run(self, timing_mode: int = 0) -> gdp_timing:
+        t = gdp_timing()
+        _check(lib().gdp_plan_run(self._h, timing_mode, ctypes.byref(t)))
+        return t
+
+    def fetch(self) -> None:
+        _check(lib().gdp_plan_fetch(self._h, self._R))
+
+    def close(self) -> None:
+        if self._h is not None and self._h.value:
+            lib().gdp_plan_destroy(self._h)
+        self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,75 @@
+"""Drop-in for the reference's compiled plugin module ``galvatron_dp_core``
+(``PYBIND11_MODULE(galvatron_dp_core, ...)``, csrc/dp_core.cpp:122-124).
+
+``DPAlg.fit`` does ``import galvatron_dp_core`` and calls
+``galvatron_dp_core.dynamic_programming_core(...)`` with eleven positional arguments
+(galvatron/core/search_engine/dynamic_programming.py:77-91).  Putting this file's directory on
+``sys.path`` ahead of the reference's ``build/lib`` makes that call run on the MI355X through
+libgalvatron_dp_hip.so; nothing else in the caller changes.
+
+Differences from the compiled reference module, all on arguments no caller reads back:
+``_mark`` and ``_f`` are filled only after ``set_export(True)`` (the argmin table lives on the
+device in a compact form, and copying L*V*S int32 back per call would dominate the run time).
+Inputs the device recurrence does not cover raise instead of computing something: NaN / -inf
+costs (``ValueError``) and a memory cost of 0 (``UnsupportedInputError``, a ``ValueError``).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from galvatron_dp import _lib
+
+__all__ = ["dynamic_programming_core", "dynamic_programming_core_batch", "set_export"]
+
+_export = False
+
+
+def set_export(flag: bool) -> None:
+    """When true, ``_f`` and ``_mark`` are written exactly as the reference writes them
+    (csrc/dp_core.cpp:61-62,72-73)."""
+    global _export
+    _export = bool(flag)
+
+
+def _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, other_mem_cost, other_time_cost,
+             export):
+    L, V, S = int(layer_num), int(max_mem), int(strategy_num)
+    mem = np.ascontiguousarray(v_data, dtype=np.int32).reshape(L, S)
+    intra = np.ascontiguousarray(intra_cost, dtype=np.float64).reshape(L, S)
+    inter = np.ascontiguousarray(inter_cost, dtype=np.float64).reshape(L, S, S)
+    keys = sorted(int(k) for k in other_mem_cost)          # std::map iterates in ascending key order
+    om = [int(other_mem_cost[k]) for k in keys]
+    ot = [float(other_time_cost[k]) if k in other_time_cost else 0.0 for k in keys]  # map::operator[] default
+    return keys, _lib.Problem(mem, intra, inter, V, om, ot, export_f=export, export_mark=export)
+
+
+def _finish(keys, prob, _mark, _f, res_list, export):
+    total_cost, remaining_mem = {}, {}
+    for i, k in enumerate(keys):
+        total_cost[k] = float(prob.total[i])
+        remaining_mem[k] = int(prob.remaining[i])
+        if prob.remaining[i] != -1:
+            res_list[k][...] = prob.res[i]                    # feasible keys only (csrc/dp_core.cpp:103-113)
+    if export:
+        np.asarray(_f)[...] = prob.f_out
+        np.asarray(_mark)[...] = prob.mark_out
+    return total_cost, remaining_mem
+
+
+def dynamic_programming_core(layer_num, max_mem, strategy_num, v_data, _mark, _f, inter_cost, intra_cost,
+                             other_mem_cost, other_time_cost, res_list):
+    """Same signature and return value as the reference (csrc/dp_core.cpp:24-35,119):
+    ``(total_cost: dict key->float, remaining_mem: dict key->int)``; ``res_list[key]`` (int32 [L],
+    pre-filled with -1 by the caller) is written in place for feasible keys."""
+    keys, prob = _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, other_mem_cost,
+                          other_time_cost, _export)
+    _lib.solve_batch([prob])
+    return _finish(keys, prob, _mark, _f, res_list, _export)
+
+
+def dynamic_programming_core_batch(calls):
+    """Many reference calls in one device batch.  ``calls`` is a sequence of 11-tuples with the
+    positional arguments of ``dynamic_programming_core``; returns the list of its return values."""
+    built = [_problem(c[0], c[1], c[2], c[3], c[6], c[7], c[8], c[9], _export) for c in calls]
+    _lib.solve_batch([b[1] for b in built])
+    return [_finish(keys, prob, c[4], c[5], c[10], _export) for (keys, prob), c in zip(built, calls)]

@@ -1,0 +1,123 @@
+/*
+ * galvatron_dp_hip.h -- C ABI of libgalvatron_dp_hip.so
+ *
+ * MI355X (gfx950) implementation of the Galvatron search engine's layer-wise
+ * dynamic program.  Every entry point below replaces, for one or many DP
+ * instances, the single reference callable
+ *
+ *     galvatron_dp_core.dynamic_programming_core(layer_num, max_mem, strategy_num,
+ *         v_data, _mark, _f, inter_cost, intra_cost,
+ *         other_mem_cost, other_time_cost, res_list)          csrc/dp_core.cpp:24-35,122-124
+ *
+ * as it is called from DPAlg.fit
+ * (galvatron/core/search_engine/dynamic_programming.py:77-91).
+ *
+ * Plain C: pointers and sizes only.  All input and output pointers are HOST
+ * memory owned by the caller and borrowed for the duration of the call (or, for
+ * a plan, until gdp_plan_create returns: inputs are copied to the device
+ * there).  The library is re-entrant: no call shares mutable state with another
+ * call, so it may be used from many threads at once (ctypes releases the GIL).
+ * There is no CPU fallback: without a usable HIP device every compute entry
+ * point fails with GDP_E_HIP.
+ */
+#ifndef GALVATRON_DP_HIP_H
+#define GALVATRON_DP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GDP_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* return codes */
+#define GDP_OK 0
+#define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S above GDP_MAX_S, ... */
+#define GDP_E_UNSUPPORTED (-2) /* an input the device recurrence does not cover: mem <= 0 */
+#define GDP_E_NONFINITE (-3)   /* NaN or -inf in a cost array (the reference's result is then order-dependent) */
+#define GDP_E_NOMEM (-4)       /* device or host allocation failed */
+#define GDP_E_HIP (-5)         /* any other HIP runtime error; text in gdp_last_error() */
+
+#define GDP_MAX_S 256 /* strategies per layer (argmin table entries are one byte) */
+
+/* gdp_problem.flags */
+#define GDP_EXPORT_F 1u    /* write result.f_out    (final f, reference layout [V][S])       */
+#define GDP_EXPORT_MARK 2u /* write result.mark_out (argmin table, reference layout [L][V][S]) */
+
+/* One DP instance == one reference call.  Field <- reference argument (csrc/dp_core.cpp:24-35):
+ *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),
+ *   S <- strategy_num, mem <- v_data, intra <- intra_cost, inter <- inter_cost,
+ *   other_mem/other_time <- other_mem_cost/other_time_cost values, in the caller's key order
+ *   (the dictionary keys themselves are never used by the arithmetic).              */
+typedef struct gdp_problem {
+    int32_t L, V, S;
+    const int32_t *mem;         /* [L][S]  memory cost in bins; every entry must be >= 1          */
+    const double *intra;        /* [L][S]                                                          */
+    const double *inter;        /* [n_inter][S][S], row = source strategy, column = target        */
+    const int32_t *inter_index; /* [L] layer -> matrix in `inter`; NULL means n_inter == L, identity */
+    int32_t n_inter;
+    int32_t n_key;              /* number of (other_mem, other_time) pairs to finish for           */
+    const int64_t *other_mem;   /* [n_key]                                                         */
+    const double *other_time;   /* [n_key]                                                         */
+    uint32_t flags;
+} gdp_problem;
+
+/* Outputs of one instance <- reference return values / written arguments (csrc/dp_core.cpp:78-119):
+ *   total[k]     <- total_cost[key k]     (+inf when infeasible)
+ *   remaining[k] <- remaining_mem[key k]  (-1 when infeasible)
+ *   res[k][0..L) <- res_list[key k]; rows of infeasible keys are left untouched, as the
+ *                   reference leaves the caller's -1 fill                          */
+typedef struct gdp_result {
+    double *total;      /* [n_key]                                   */
+    int32_t *remaining; /* [n_key]                                   */
+    int32_t *res;       /* [n_key][L]                                */
+    double *f_out;      /* [V][S]    or NULL (needs GDP_EXPORT_F)    */
+    int32_t *mark_out;  /* [L][V][S] or NULL (needs GDP_EXPORT_MARK) */
+} gdp_result;
+
+/* Device-side timings of one gdp_plan_run, taken with HIP events on the plan's stream. */
+typedef struct gdp_timing {
+    float total_ms;        /* first kernel to last kernel (relaxation layers + epilogue)      */
+    float relax_ms;        /* sum of the per-launch durations of the relaxation kernel         */
+    int32_t relax_launches;
+    int32_t reserved;
+    double relaxations;    /* sum over instances of L*V*S*S                                    */
+    double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write) */
+} gdp_timing;
+
+typedef struct gdp_plan gdp_plan;
+
+/* Solve one instance: validate, upload, run, download.  Replaces one
+ * dynamic_programming_core call (csrc/dp_core.cpp:24-120). */
+int gdp_solve(const gdp_problem *p, gdp_result *r);
+
+/* Solve n independent instances (e.g. every pipeline stage of every pp_deg, or a whole
+ * bsz x chunk sweep: the DPAlg.fit calls issued from dynamic_programming.py:446-488 and
+ * search_engine.py:477-498) with one launch grid per layer index. */
+int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r);
+
+/* The same in three steps, so that a caller (or a benchmark) can keep inputs resident in
+ * device memory and run the device part repeatedly:
+ *   create  -- validate + allocate + copy inputs to the device
+ *   run     -- layer kernels + on-device backtrack; timing may be NULL.
+ *              timing_mode 0: none, 1: total_ms only, 2: also per-launch relaxation events
+ *   fetch   -- copy results of the last run to the caller's arrays
+ *   destroy -- release everything                                              */
+int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out);
+int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing);
+int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r);
+void gdp_plan_destroy(gdp_plan *plan);
+
+/* Text of the calling thread's last error ("" if none). */
+const char *gdp_last_error(void);
+/* GDP_VERSION of the built library. */
+int gdp_version(void);
+/* Writes "name;arch;CUs;HBM bytes" of the current device into buf; GDP_E_HIP without a device. */
+int gdp_device_info(char *buf, size_t len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GALVATRON_DP_HIP_H */

@@ -1,0 +1,160 @@
+"""Writes tests/golden/dp_core_golden.json from the reference's compiled dp_core.
+
+Run in the build container only (it needs oracle/_ref, i.e. /root/reference):
+
+    python oracle/build.py && python tests/golden/make_golden.py [--only NAME ...] [--jobs N]
+
+For every case the seeded generator (galvatron_dp.workloads) rebuilds the inputs, the
+reference's ``dynamic_programming_core`` (csrc/dp_core.cpp:24-120, compiled by
+oracle/build.py) solves them exactly as ``DPAlg.fit`` calls it, and the fixture keeps
+only data: the generator call, a SHA-256 of the input bytes, the per-key total cost
+(hex float), strategy list and remaining memory, and SHA-256 digests of the final ``f``
+[V,S] f64 and ``mark`` [L,V,S] int32 arrays in the reference's layouts.
+"""
+from __future__ import annotations
+
+import argparse
+import hashlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "hetu-galvatron_amd"))
+
+from galvatron_dp import workloads as W  # noqa: E402
+
+OUT = os.path.join(HERE, "dp_core_golden.json")
+
+
+def cases():
+    """name -> (builder name, kwargs).  Builders are looked up in ``golden_cases``."""
+    c = {}
+    c["cfg0"] = ("config0", {})
+    c["cfg0_other_time"] = ("config0", {"random_other_time": True})
+    c["cfg1"] = ("config1", {})
+    c["cfg2"] = ("config2", {})
+    c["cfg2_small"] = ("config2", {"L": 12, "S": 64, "V": 12288})
+    c["cfg4"] = ("config4", {})
+    c["cfg4_small"] = ("config4", {"V": 16384, "n_each": 5})
+    for i in range(256):
+        c[f"cfg3_{i:03d}"] = ("config3_item", {"i": i})
+    for i in range(8):
+        c[f"cfg3_smallV_{i}"] = ("config3_item", {"i": 35 * i + 3, "V": 8192})
+    # tie-heavy and edge cases (small enough for the CPU suite)
+    for i, (L, S, V) in enumerate([(6, 5, 300), (9, 22, 700), (5, 64, 500), (4, 65, 400), (7, 3, 257),
+                                   (3, 127, 300), (12, 44, 1500), (2, 1, 64), (1, 7, 100), (5, 88, 640)]):
+        c[f"ties_{i}"] = ("ties", {"seed": 1000 + i, "L": L, "S": S, "V": V})
+        c[f"rand_{i}"] = ("rand", {"seed": 2000 + i, "L": L, "S": S, "V": V})
+        c[f"infeasible_{i}"] = ("infeasible", {"seed": 3000 + i, "L": L, "S": S, "V": V})
+    c["galvatron_like"] = ("galvatron_like", {})
+    return c
+
+
+def build_case(builder: str, kw: dict) -> W.Instance:
+    if builder == "config3_item":
+        kw = dict(kw)
+        i = kw.pop("i")
+        return W.config3(n_limit=i + 1, **kw)[i]
+    if builder == "ties":
+        rng = np.random.Generator(np.random.PCG64(kw["seed"]))
+        inst = W.random_instance(rng, kw["L"], kw["S"], kw["V"], integer_costs=True,
+                                 mem_hi=max(1, kw["V"] // (kw["L"] + 1)), per_layer_inter=bool(kw["seed"] % 2))
+        # duplicate a strategy so that exact ties between columns exist
+        if kw["S"] >= 3:
+            inst.mem[:, -1] = inst.mem[:, 0]
+            inst.intra[:, -1] = inst.intra[:, 0]
+            inter = np.array(inst.inter)
+            inter[:, -1, :] = inter[:, 0, :]
+            inter[:, :, -1] = inter[:, :, 0]
+            inst.inter = inter
+            inst.inter_tables, inst.inter_index = inter, np.arange(kw["L"], dtype=np.int32)
+        return inst
+    if builder == "rand":
+        rng = np.random.Generator(np.random.PCG64(kw["seed"]))
+        return W.random_instance(rng, kw["L"], kw["S"], kw["V"], mem_hi=max(1, kw["V"] // max(2, kw["L"] - 1)))
+    if builder == "infeasible":
+        rng = np.random.Generator(np.random.PCG64(kw["seed"]))
+        return W.random_instance(rng, kw["L"], kw["S"], kw["V"], mem_hi=max(1, kw["V"] // (kw["L"] + 1)),
+                                 inf_frac=0.2, over_frac=0.15, n_keys=4)
+    if builder == "galvatron_like":
+        return galvatron_like()
+    return getattr(W, builder)(**kw)
+
+
+def galvatron_like() -> W.Instance:
+    """Shape of a real search-engine call: 28 identical layers, inter made of zeros and
+    the 1e-10..3e-9 ordering sentinels, first layer's inter zeroed, four keys
+    (dynamic_programming.py:241,266,347-372).  Numbers are synthetic."""
+    rng = np.random.Generator(np.random.PCG64(77))
+    L, S, V = 28, 40, 29493
+    mem_row = rng.integers(300, 2600, size=S)
+    t_row = np.round(rng.uniform(20, 60, size=S), 3)
+    m = np.zeros((S, S))
+    sent = np.array([0.0, 1e-10, 1e-9, 2e-9, 3e-9, 0.37, 1.21])
+    m[:] = sent[rng.integers(0, len(sent), size=(S, S))]
+    np.fill_diagonal(m, 0.0)
+    inter = np.repeat(m[None], L, 0)
+    inter[0] = 0.0
+    om = {1: 4100, 2: 2300, 4: 1500, 8: 900}
+    ot = {1: 31.5, 2: 17.25, 4: 9.125, 8: 6.0625}
+    return W.Instance("galvatron_like", np.repeat(mem_row[None], L, 0).astype(np.int32),
+                      np.repeat(t_row[None], L, 0), inter, V, om, ot, inter, np.arange(L, dtype=np.int32))
+
+
+def solve_case(item):
+    name, (builder, kw) = item
+    from oracle import dp_oracle as O
+    inst = build_case(builder, kw)
+    t0 = time.time()
+    total, res, rem, f, mark = O.ref_solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem,
+                                           inst.other_time, keep=True)
+    dt = time.time() - t0
+    keys = sorted(total)
+    rec = {
+        "builder": builder, "kwargs": kw, "L": inst.L, "S": inst.S, "V": inst.V,
+        "input_sha256": inst.digest(), "keys": keys,
+        "total_hex": [float(total[k]).hex() for k in keys],
+        "remaining": [int(rem[k]) for k in keys],
+        "res": [res[k] for k in keys],
+        "f_sha256": hashlib.sha256(f.tobytes()).hexdigest(),
+        "mark_sha256": hashlib.sha256(mark.tobytes()).hexdigest(),
+        "ref_seconds": round(dt, 3),
+    }
+    print(f"{name}: {dt:.1f}s", flush=True)
+    return name, rec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--only", nargs="*", default=None, help="case-name prefixes to (re)generate")
+    ap.add_argument("--jobs", type=int, default=1)
+    a = ap.parse_args()
+    todo = cases()
+    if a.only:
+        todo = {k: v for k, v in todo.items() if any(k.startswith(p) for p in a.only)}
+    gold = {}
+    if os.path.exists(OUT):
+        with open(OUT) as fh:
+            gold = json.load(fh)
+    if a.jobs > 1:
+        import multiprocessing as mp
+        with mp.get_context("fork").Pool(a.jobs) as pool:
+            for name, rec in pool.imap_unordered(solve_case, list(todo.items())):
+                gold[name] = rec
+    else:
+        for item in todo.items():
+            name, rec = solve_case(item)
+            gold[name] = rec
+    with open(OUT, "w") as fh:
+        json.dump({k: gold[k] for k in sorted(gold)}, fh, indent=0, separators=(",", ":"))
+    print("wrote", OUT, len(gold), "cases")
+
+
+if __name__ == "__main__":
+    main()
