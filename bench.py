@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Benchmark of the layer-wise DP hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg0|cfg1|cfg4]
+
+One "step" is one complete solve of the workload on the device: every layer's relaxation kernel
+over every instance of the batch, plus the on-device backtrack, with the inputs already resident
+in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
+
+* ``value``        min-plus relaxations per second, sum over instances of L*V*S*S divided by the
+                   wall time of the timed steps (host clock around K steps, device synchronised on
+                   both sides).
+* ``roofline``     for the relaxation kernel (the only kernel that matters): 3 fp64 vector
+                   operations (two additions, one comparison) per relaxation, divided by the average
+                   launch duration measured with HIP events on the stream the kernel runs on;
+                   peak = 39.3 TFLOP/s = MI355X's published 78.6 TFLOP/s fp64 vector rate, which
+                   counts an FMA as two operations -- additions and comparisons cannot fuse.
+                   ``roofline_hbm`` is the same launch against 8 TB/s with the algorithmic bytes
+                   V*S*(8 read + 8 write + 1 argmin) per layer and instance.
+* ``cpu_baseline`` the reference's own dp_core (compiled into oracle/_ref by oracle/build.py) or,
+                   where that file is absent, the C restatement in oracle/, timed on this host on a
+                   bounded sample of the same workload (its first layers), one thread.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "hetu-galvatron_amd"))
+
+PEAK_FP64_VALU_TFLOPS = 39.3   # 78.6 TFLOP/s published (FMA = 2 ops) / 2
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the relaxation kernel measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE (scaled by a copy kernel of known size); see profiles/.  None until measured.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
+
+
+def _problems(workload: str):
+    from galvatron_dp import _lib, workloads as W
+    if workload == "cfg3":
+        insts = W.config3()
+    else:
+        insts = [W.CONFIGS[int(workload[3:])]()]
+    probs = []
+    for inst in insts:
+        keys = sorted(inst.other_mem)
+        probs.append(_lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V,
+                                  [inst.other_mem[k] for k in keys], [inst.other_time[k] for k in keys],
+                                  inter_index=inst.inter_index))
+    return insts, probs
+
+
+def _cpu_baseline(workload: str, budget_s: float = 20.0):
+    """Reference dp_core (or the C port) on the first layers of the workload's first instance."""
+    import numpy as np
+    from galvatron_dp import workloads as W
+    from oracle import dp_oracle as O
+    inst = W.config3(n_limit=1)[0] if workload == "cfg3" else W.CONFIGS[int(workload[3:])]()
+    use_ref = O.ref_available()
+    rate_guess = 4.0e8 if use_ref else 5.5e8
+    per_layer = inst.V * inst.S * inst.S
+    n_layers = int(max(1, min(inst.L, budget_s * rate_guess // per_layer)))
+    mem, intra, inter = inst.mem[:n_layers], inst.intra[:n_layers], np.ascontiguousarray(inst.inter[:n_layers])
+    fn = O.ref_solve if use_ref else O.solve
+    t0 = time.perf_counter()
+    fn(mem, intra, inter, inst.V, inst.other_mem, inst.other_time)
+    dt = time.perf_counter() - t0
+    relax = n_layers * per_layer
+    return {"value": relax / dt, "unit": "relaxations/s", "cores": 1,
+            "kind": "reference" if use_ref else "port",
+            "sample": f"first {n_layers} of {inst.L} layers of {inst.name} (V={inst.V}, S={inst.S}), "
+                      f"{relax:.3g} relaxations in {dt:.2f} s, single thread, includes the host argmin-table "
+                      f"allocation the reference caller does"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--also", default="cfg3", help="comma-separated extra workloads summarised in the same line")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs the DP hot path on ONE GPU; --gpus must be 1 "
+              "(instances of a batch are independent and would shard by instance, see DESIGN.md)", file=sys.stderr)
+        return 2
+
+    import ctypes
+
+    from galvatron_dp import _lib
+    _lib.lib()                                        # fails loudly when the HIP library is missing
+    hip = ctypes.CDLL("libamdhip64.so")               # already mapped by the library above
+
+    def device_sync():
+        if hip.hipDeviceSynchronize() != 0:
+            raise RuntimeError("hipDeviceSynchronize failed")
+
+    def measure(workload, steps, warmup):
+        insts, probs = _problems(workload)
+        with _lib.Plan(probs) as plan:
+            for _ in range(warmup):
+                plan.run(0)
+            device_sync()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                plan.run(0)                       # synchronises the plan's stream before returning
+            device_sync()
+            wall = time.perf_counter() - t0
+            tm = plan.run(2)                       # per-launch HIP events on the plan's stream
+            t1 = plan.run(1)
+            plan.fetch()
+        relax = tm.relaxations
+        launches = tm.relax_launches
+        avg_launch_s = tm.relax_ms * 1e-3 / launches
+        return {
+            "insts": insts, "probs": probs, "relaxations": relax, "ms_per_step": wall / steps * 1e3,
+            "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
+            "device_ms": t1.total_ms,
+            "tflops": 3.0 * relax / launches / avg_launch_s / 1e12,
+            "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
+            "bytes_per_launch": tm.relax_bytes / launches,
+        }
+
+    m = measure(a.workload, a.steps, a.warmup)
+    insts = m["insts"]
+    first = insts[0]
+    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(a.workload)
+    line = {
+        "metric": "min-plus relaxations/s (L*V*S^2)", "value": m["value"], "unit": "relaxations/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": m["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
+                   "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
+                   "mark_bytes": 1, "search_wall_ms_device": m["device_ms"], "device": _lib.device_info()},
+        "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
+                     "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,
+                     "kernel": "gdp_relax_kernel", "launches_per_step": m["launches"],
+                     "avg_launch_ms": m["avg_launch_ms"], "flops_per_relaxation": 3},
+        "roofline_hbm": {"bound": "hbm", "achieved": m["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": m["gbs"] / PEAK_HBM_GBS, "traffic": traffic,
+                         "algorithmic_bytes_per_launch": m["bytes_per_launch"]},
+    }
+    also = {}
+    for w in [x for x in a.also.split(",") if x and x != a.workload]:
+        mm = measure(w, max(3, a.steps // 4), 1)
+        also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
+                   "roofline_frac_valu_fp64": mm["tflops"] / PEAK_FP64_VALU_TFLOPS,
+                   "roofline_frac_hbm": mm["gbs"] / PEAK_HBM_GBS, "avg_launch_ms": mm["avg_launch_ms"]}
+    if also:
+        line["also"] = also
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = _cpu_baseline(a.workload)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,75 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every symbol the header
+declares, and the host-side argument handling behaves (no compute call is made here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from galvatron_dp import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "galvatron_dp_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gdp_[a-z_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    lib = _lib.lib()
+    names = _declared_symbols()
+    assert set(names) == set(_lib.EXPORTED_SYMBOLS), names
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_version_and_struct_sizes():
+    assert _lib.lib().gdp_version() == 100
+    assert ctypes.sizeof(_lib.gdp_problem) == 80
+    assert ctypes.sizeof(_lib.gdp_result) == 40
+    assert ctypes.sizeof(_lib.gdp_timing) == 32
+
+
+def test_validation_happens_before_any_device_work():
+    # these are rejected on the host, so they behave the same with or without a GPU
+    lib = _lib.lib()
+    mem = np.ones((2, 3), np.int32)
+    intra = np.ones((2, 3))
+    inter = np.zeros((2, 3, 3))
+
+    def rc_of(p):
+        h = ctypes.c_void_p()
+        P = (ctypes.POINTER(_lib.gdp_problem) * 1)(ctypes.pointer(p._c_problem))
+        return lib.gdp_plan_create(1, P, ctypes.byref(h)), lib.gdp_last_error().decode()
+
+    m0 = mem.copy(); m0[1, 1] = 0
+    rc, msg = rc_of(_lib.Problem(m0, intra, inter, 10, [0], [0.0]))
+    assert rc == _lib.GDP_E_UNSUPPORTED and "0" in msg
+    mn = mem.copy(); mn[0, 0] = -3
+    assert rc_of(_lib.Problem(mn, intra, inter, 10, [0], [0.0]))[0] == _lib.GDP_E_BADARG
+    bad = intra.copy(); bad[0, 2] = np.nan
+    assert rc_of(_lib.Problem(mem, bad, inter, 10, [0], [0.0]))[0] == _lib.GDP_E_NONFINITE
+    bad = inter.copy(); bad[1, 2, 0] = -np.inf
+    assert rc_of(_lib.Problem(mem, intra, bad, 10, [0], [0.0]))[0] == _lib.GDP_E_NONFINITE
+    huge = intra.copy(); huge[:] = 1e300
+    assert rc_of(_lib.Problem(mem, huge, inter, 10, [0], [0.0]))[0] == _lib.GDP_E_NONFINITE
+    big_s = np.ones((1, _lib.GDP_MAX_S + 1), np.int32)
+    p = _lib.Problem(big_s, np.ones((1, _lib.GDP_MAX_S + 1)), np.zeros((1, _lib.GDP_MAX_S + 1, _lib.GDP_MAX_S + 1)),
+                     10, [0], [0.0])
+    assert rc_of(p)[0] == _lib.GDP_E_BADARG
+    assert lib.gdp_plan_create(0, None, ctypes.byref(ctypes.c_void_p())) == _lib.GDP_E_BADARG
+
+
+def test_problem_shape_checks():
+    with pytest.raises(ValueError):
+        _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 4)), np.zeros((2, 3, 3)), 10, [0], [0.0])
+    with pytest.raises(ValueError):
+        _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 3)), np.zeros((1, 3, 3)), 10, [0], [0.0])
+    with pytest.raises(ValueError):
+        _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 3)), np.zeros((2, 3, 3)), 10, [0, 1], [0.0])
+    p = _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 3)), np.zeros((1, 3, 3)), 10, [0], [0.0],
+                     inter_index=[0, 0])
+    assert p.relaxations == 2 * 10 * 9
