@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -40,20 +41,40 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct HostInst {
     int orig;  // index in the caller's arrays
-    int L, V, S, SP, P, ntile, n_key, n_inter;
+    int L, V, S, SP, SU, P, ntile, n_key, n_inter, variant, nbuf;
     int64_t ld, ldm;
     uint32_t flags;
     int key_begin;  // first entry in the key table
     int res_begin;  // first element in the result array
     // byte offsets inside the device allocation
-    size_t off_H0, off_H1, off_M, off_inter, off_intra, off_index, off_roff, off_mem;
+    size_t off_H, off_M, off_inter, off_intra, off_index, off_roff, off_mem, off_dep;
 };
 
 struct Group {  // instances with the same S, sorted by L descending
-    int first, count, SP, S, max_L, max_ntile;
+    int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt, grid_blocks;
     int64_t max_ld;
     std::vector<int> active;  // active[l] = number of instances with L > l
+    size_t off_sched, off_active, off_next, off_cnt;  // byte offsets in the device allocation
 };
+
+// Target-tile width: the one that pads S the least (ties: the first).
+int pick_ts(int S)
+{
+    int best = GDP_VARIANTS[0].ts;
+    size_t best_sp = align_up((size_t)S, (size_t)best);
+    for (int v = 1; v < GDP_NUM_VARIANTS; ++v) {
+        const size_t sp = align_up((size_t)S, (size_t)GDP_VARIANTS[v].ts);
+        if (sp < best_sp) { best = GDP_VARIANTS[v].ts; best_sp = sp; }
+    }
+    return best;
+}
+
+int find_variant(int ts, int r)
+{
+    for (int v = 0; v < GDP_NUM_VARIANTS; ++v)
+        if (GDP_VARIANTS[v].ts == ts && GDP_VARIANTS[v].r == r) return v;
+    return -1;
+}
 
 }  // namespace
 
@@ -75,6 +96,16 @@ struct gdp_plan {
     std::vector<int32_t> h_res;
     double relaxations = 0, relax_bytes = 0;
     bool ran = false;
+    bool fused = true;            // one launch for all layers (work queue) instead of one per layer
+    int64_t spin_limit = 1 << 22; // polls a waiting wave makes before the launch is abandoned
+    size_t off_zero = 0, zero_words = 0, off_abort = 0;
+    int num_cu = 0;
+    bool can_fuse = true;    // cost buffers were laid out one per layer
+    bool rezero = false;     // buffer 0 is overwritten during a run and must be zeroed before each
+    bool fused_gave_up = false;  // a fused launch was abandoned and the plan switched to per-layer launches
+    bool no_fallback = false;    // GDP_OPT_NO_FALLBACK: report that instead of switching (tests)
+    int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
+    bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
 
 namespace {
@@ -151,14 +182,27 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
 {
     pl->n = n;
     GDP_HIP(hipGetDevice(&pl->device));
+    // defaults of the plan options can be preset from the environment
+    if (const char *e = getenv("GALVATRON_DP_FUSED")) pl->fused = atoi(e) != 0;
+    if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
+    if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
+    if (const char *e = getenv("GALVATRON_DP_SPIN_LIMIT")) {
+        const long long v = atoll(e);
+        if (v >= 1) pl->spin_limit = v;
+    }
     // ---- shapes -------------------------------------------------------------------------------
+    {
+        hipDeviceProp_t prop;
+        GDP_HIP(hipGetDeviceProperties(&prop, pl->device));
+        pl->num_cu = prop.multiProcessorCount;
+    }
     std::vector<HostInst> inst((size_t)n);
     for (int i = 0; i < n; ++i) {
         const gdp_problem *q = p[i];
         HostInst &h = inst[(size_t)i];
         h.orig = i;
         h.L = q->L; h.V = q->V; h.S = q->S;
-        h.SP = (int)align_up((size_t)q->S, GDP_TS);
+        h.SU = (int)align_up((size_t)q->S, GDP_SRC_UNROLL);
         h.n_key = q->n_key;
         h.n_inter = q->inter_index ? q->n_inter : q->L;
         h.flags = q->flags;
@@ -166,30 +210,57 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         for (size_t k = 0; k < (size_t)q->L * q->S; ++k)
             if (q->mem[k] < q->V) maxm = std::max(maxm, q->mem[k]);
         h.P = (int)align_up((size_t)std::max(maxm, 1), 64);
-        h.ntile = (q->V + GDP_TILE_ROWS - 1) / GDP_TILE_ROWS;
-        h.ldm = (int64_t)h.ntile * GDP_TILE_ROWS;
-        h.ld = h.P + h.ldm;
     }
     // group by S, then by L descending (stable, so equal shapes keep the caller's order)
     std::stable_sort(inst.begin(), inst.end(), [](const HostInst &a, const HostInst &b) {
         if (a.S != b.S) return a.S < b.S;
         return a.L > b.L;
     });
+    const int64_t wave_slots = (int64_t)pl->num_cu * 4 * 4;  // 4 SIMDs x 4 resident waves
     for (int i = 0; i < n;) {
         Group g;
-        g.first = i; g.S = inst[(size_t)i].S; g.SP = inst[(size_t)i].SP;
-        g.max_L = 0; g.max_ntile = 0; g.max_ld = 0;
+        g.first = i; g.S = inst[(size_t)i].S;
         int j = i;
-        while (j < n && inst[(size_t)j].S == g.S) {
-            g.max_L = std::max(g.max_L, inst[(size_t)j].L);
-            g.max_ntile = std::max(g.max_ntile, inst[(size_t)j].ntile);
-            g.max_ld = std::max(g.max_ld, inst[(size_t)j].ld);
-            ++j;
-        }
+        while (j < n && inst[(size_t)j].S == g.S) ++j;
         g.count = j - i;
+        // Register tile.  Width: least padding of S.  Height: the tallest whose first layer still
+        // gives every resident wave at least two tasks, so that the stores of one task drain under
+        // the arithmetic of the next; small problems get the shortest (most parallel) one.
+        const int ts = pick_ts(g.S);
+        const int ntb = (int)align_up((size_t)g.S, (size_t)ts) / ts;
+        int best_r = 0;
+        {
+            // variants of one width are listed tallest first
+            for (int v = 0; v < GDP_NUM_VARIANTS; ++v) {
+                if (GDP_VARIANTS[v].ts != ts) continue;
+                const int r = GDP_VARIANTS[v].r;
+                int64_t tasks = 0;
+                for (int k = i; k < j; ++k) tasks += ((int64_t)inst[(size_t)k].V + 64 * r - 1) / (64 * r) * ntb;
+                best_r = r;
+                if (tasks >= 2 * wave_slots) break;
+            }
+        }
+        if (pl->tile_r_override > 0 && find_variant(ts, pl->tile_r_override) >= 0) best_r = pl->tile_r_override;
+        g.variant = find_variant(ts, best_r);
+        const int tile_rows = 64 * best_r;
+        g.SP = ntb * ts;
+        g.ntb = ntb;
+        g.max_L = 0; g.max_ntile = 0; g.max_ld = 0;
+        for (int k = i; k < j; ++k) {
+            HostInst &h = inst[(size_t)k];
+            h.variant = g.variant;
+            h.SP = g.SP;
+            h.ntile = (h.V + tile_rows - 1) / tile_rows;
+            h.ldm = (int64_t)align_up((size_t)h.ntile * tile_rows, 256);
+            h.ld = h.P + h.ldm;
+            g.max_L = std::max(g.max_L, h.L);
+            g.max_ntile = std::max(g.max_ntile, h.ntile);
+            g.max_ld = std::max(g.max_ld, h.ld);
+        }
         g.active.assign((size_t)g.max_L, 0);
         for (int k = i; k < j; ++k)
             for (int l = 0; l < inst[(size_t)k].L; ++l) g.active[(size_t)l]++;
+        g.nbt = (g.max_ntile * g.ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
         pl->max_L = std::max(pl->max_L, g.max_L);
         pl->groups.push_back(g);
         i = j;
@@ -211,29 +282,54 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     pl->n_res_total = nres;
     pl->off_insts = take(sizeof(GdpDevInst) * (size_t)n);
     pl->off_keys = take(sizeof(GdpDevKey) * (size_t)std::max(nk, 1));
+    for (auto &g : pl->groups) {
+        g.off_sched = take(sizeof(GdpSched));
+        g.off_active = take(sizeof(int32_t) * (size_t)g.max_L);
+    }
     for (auto &h : inst) {
-        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.S + 1) * h.SP);
+        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_UNROLL) * h.SP);
         h.off_intra = take(sizeof(double) * (size_t)h.L * h.SP);
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
-        h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.S + 1));
+        h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_UNROLL));
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
+        h.off_dep = take(sizeof(int32_t) * (size_t)h.L);
     }
     const size_t small_bytes = off;
+    // words that every run resets to zero: abort flag, ticket counters, completion counters
+    pl->off_zero = off;
+    pl->off_abort = take(sizeof(int32_t));
+    for (auto &g : pl->groups) {
+        g.off_next = take(sizeof(int32_t) * (size_t)g.max_L * GDP_QUEUES);
+        g.off_cnt = take(sizeof(int32_t) * (size_t)g.count * g.max_L * g.max_ntile);
+    }
+    pl->zero_words = (off - pl->off_zero) / sizeof(int32_t);
     pl->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(nk, 1));
     pl->off_res = take(sizeof(int32_t) * std::max<size_t>(nres, 1));
-    for (auto &h : inst) {
-        h.off_H0 = take(sizeof(double) * (size_t)(h.S + 1) * (size_t)h.ld);
-        h.off_H1 = take(sizeof(double) * (size_t)(h.S + 1) * (size_t)h.ld);
-        h.off_M = take((size_t)h.L * h.S * (size_t)h.ldm);
-    }
-    pl->dbytes = off;
-    {
-        hipError_t e = hipMalloc((void **)&pl->dbase, pl->dbytes);
-        if (e != hipSuccess) {
-            char buf[128];
-            snprintf(buf, sizeof buf, "hipMalloc of %zu bytes", pl->dbytes);
-            return fail_hip(e, buf);
+    const size_t fixed_bytes = off;
+    // One cost buffer per layer lets all layers share a launch; if that does not fit in device
+    // memory, fall back to two buffers and one launch per layer.
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        off = fixed_bytes;
+        pl->can_fuse = pl->fused;
+        pl->rezero = false;
+        for (auto &h : inst) {
+            h.nbuf = pl->fused ? h.L + 1 : 2;
+            if (h.nbuf < h.L + 1) pl->rezero = true;
+            h.off_H = take(sizeof(double) * (size_t)h.nbuf * (size_t)(h.S + 1) * (size_t)h.ld);
+            h.off_M = take((size_t)h.L * h.S * (size_t)h.ldm);
         }
+        pl->dbytes = off;
+        hipError_t e = hipMalloc((void **)&pl->dbase, pl->dbytes);
+        if (e == hipSuccess) break;
+        pl->dbase = nullptr;
+        (void)hipGetLastError();
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->fused) {
+            pl->fused = false;
+            continue;
+        }
+        char buf[128];
+        snprintf(buf, sizeof buf, "hipMalloc of %zu bytes", pl->dbytes);
+        return fail_hip(e, buf);
     }
     // ---- build the small region on the host ------------------------------------------------------
     std::vector<char> stage;
@@ -248,22 +344,25 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         const HostInst &h = inst[(size_t)i];
         const gdp_problem *q = p[h.orig];
         GdpDevInst &d = di[i];
-        d.H[0] = reinterpret_cast<double *>(pl->dbase + h.off_H0);
-        d.H[1] = reinterpret_cast<double *>(pl->dbase + h.off_H1);
+        d.H = reinterpret_cast<double *>(pl->dbase + h.off_H);
+        d.hstride = (int64_t)(h.S + 1) * h.ld;
+        d.nbuf = h.nbuf;
         d.M = reinterpret_cast<uint8_t *>(pl->dbase + h.off_M);
         d.inter = reinterpret_cast<const double *>(pl->dbase + h.off_inter);
         d.intra = reinterpret_cast<const double *>(pl->dbase + h.off_intra);
         d.inter_index = reinterpret_cast<const int32_t *>(pl->dbase + h.off_index);
         d.roff = reinterpret_cast<const int64_t *>(pl->dbase + h.off_roff);
         d.mem = reinterpret_cast<const int32_t *>(pl->dbase + h.off_mem);
+        d.dep = reinterpret_cast<const int32_t *>(pl->dbase + h.off_dep);
         d.ld = h.ld; d.ldm = h.ldm;
-        d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.P = h.P; d.ntile = h.ntile;
-        d.pad0 = d.pad1 = 0;
-        // inter: [T][S+1][SP], zero padded
+        d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.SU = h.SU; d.P = h.P; d.ntile = h.ntile;
+        const int rows = h.SU + GDP_SRC_UNROLL;  // source rows per matrix / offsets per layer
+        const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
+        // inter: [T][rows][SP], zero padded
         double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
         for (int t = 0; t < h.n_inter; ++t)
             for (int a = 0; a < h.S; ++a)
-                memcpy(it + ((size_t)t * (h.S + 1) + a) * h.SP, q->inter + ((size_t)t * h.S + a) * h.S,
+                memcpy(it + ((size_t)t * rows + a) * h.SP, q->inter + ((size_t)t * h.S + a) * h.S,
                        sizeof(double) * (size_t)h.S);
         double *ia = reinterpret_cast<double *>(stage.data() + h.off_intra);
         for (int l = 0; l < h.L; ++l)
@@ -275,7 +374,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         int64_t *ro = reinterpret_cast<int64_t *>(stage.data() + h.off_roff);
         const int64_t inf_row = (int64_t)h.S * h.ld + h.P;
         for (int l = 0; l <= h.L; ++l) {
-            int64_t *row = ro + (size_t)l * (h.S + 1);
+            int64_t *row = ro + (size_t)l * rows;
             for (int s = 0; s < h.S; ++s) {
                 if (l == 0) {
                     row[s] = (int64_t)s * h.ld + h.P;  // zeros: the caller's initial f
@@ -284,7 +383,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
                     row[s] = (m >= h.V) ? inf_row : (int64_t)s * h.ld + h.P - m;
                 }
             }
-            row[h.S] = row[0];  // target of the last prefetch
+            for (int s = h.S; s < rows; ++s) row[s] = inf_row;  // padding sources and prefetch targets
+        }
+        // dep[l]: a reader of layer l's output at tile t touches tiles [t - dep[l], t]
+        int32_t *dep = reinterpret_cast<int32_t *>(stage.data() + h.off_dep);
+        for (int l = 0; l < h.L; ++l) {
+            int maxm = 0;
+            for (int s = 0; s < h.S; ++s) {
+                const int m = q->mem[(size_t)l * h.S + s];
+                if (m < h.V) maxm = std::max(maxm, m);
+            }
+            dep[l] = (maxm + tile_rows - 1) / tile_rows;
         }
         for (int k = 0; k < h.n_key; ++k) {
             GdpDevKey &key = dk[h.key_begin + k];
@@ -296,10 +405,39 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         pl->relaxations += (double)h.L * h.V * (double)h.S * h.S;
         pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + 1);
     }
+    for (auto &g : pl->groups) {
+        GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
+        sc->next = reinterpret_cast<int32_t *>(pl->dbase + g.off_next);
+        sc->cnt = reinterpret_cast<int32_t *>(pl->dbase + g.off_cnt);
+        sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
+        sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
+        sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb; sc->nbt = g.nbt;
+        sc->spin_limit = pl->spin_limit;
+        int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
+        int64_t tasks = 0;
+        for (int l = 0; l < g.max_L; ++l) {
+            act[l] = g.active[(size_t)l];
+            tasks += (int64_t)g.active[(size_t)l] * g.nbt;
+        }
+        int per_cu = 1;
+        GDP_HIP(gdp_fused_blocks_per_cu(g.variant, &per_cu));
+        const int64_t first_layer = (int64_t)g.active[0] * g.nbt;
+        int want = 4;  // resident blocks per CU (16 waves, 4 per SIMD)
+        if (const char *e = getenv("GALVATRON_DP_BLOCKS_PER_CU")) want = std::max(1, atoi(e));
+        int64_t grid = std::min<int64_t>(first_layer, (int64_t)std::max(std::min(per_cu, want), 1) * pl->num_cu);
+        g.grid_blocks = (int)std::max<int64_t>(GDP_QUEUES, grid / GDP_QUEUES * GDP_QUEUES);
+        (void)tasks;
+    }
     GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));
     GDP_HIP(hipEventCreate(&pl->ev_begin));
     GDP_HIP(hipEventCreate(&pl->ev_end));
     GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
+    {   // the parts of the cost buffers that no run ever overwrites
+        const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
+        for (const Group &g : pl->groups)
+            GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, GDP_INIT_PADS | GDP_INIT_ZERO,
+                                    pl->stream));
+    }
     GDP_HIP(hipStreamSynchronize(pl->stream));
     pl->inst.swap(inst);
     pl->h_out.resize((size_t)std::max(nk, 1));
@@ -315,7 +453,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
     int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
     size_t launches = 0;
-    for (const Group &g : pl->groups) launches += (size_t)g.max_L;
+    for (const Group &g : pl->groups) launches += pl->fused ? 1 : (size_t)g.max_L;
     if (mode >= 2)
         while (pl->ev_relax.size() < 2 * launches) {
             hipEvent_t e;
@@ -323,20 +461,51 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
             pl->ev_relax.push_back(e);
         }
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_begin, pl->stream));
-    for (const Group &g : pl->groups)
-        GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, pl->stream));
+    {
+        const int what = (pl->rezero ? GDP_INIT_ZERO : 0) | (pl->poison ? GDP_INIT_POISON : 0);
+        if (what)
+            for (const Group &g : pl->groups)
+                GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, what, pl->stream));
+    }
     size_t li = 0;
-    for (int l = 0; l < pl->max_L; ++l)
+    if (pl->fused) {
+        GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
+                                pl->stream));
         for (const Group &g : pl->groups) {
-            if (l >= g.max_L) continue;
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-            GDP_HIP(gdp_launch_relax(d_insts + g.first, g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
+            GDP_HIP(gdp_launch_relax_fused(g.variant, d_insts + g.first,
+                                           reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), g.grid_blocks,
+                                           pl->stream));
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
             ++li;
         }
+    } else {
+        for (int l = 0; l < pl->max_L; ++l)
+            for (const Group &g : pl->groups) {
+                if (l >= g.max_L) continue;
+                if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
+                GDP_HIP(gdp_launch_relax(g.variant, d_insts + g.first, g.active[(size_t)l], g.max_ntile, g.SP, l,
+                                         pl->stream));
+                if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
+                ++li;
+            }
+    }
     GDP_HIP(gdp_launch_epilogue(d_insts, d_keys, pl->n_key_total, d_out, d_res, pl->stream));
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
+    int32_t aborted = 0;
+    if (pl->fused)
+        GDP_HIP(hipMemcpyAsync(&aborted, pl->dbase + pl->off_abort, sizeof aborted, hipMemcpyDeviceToHost, pl->stream));
     GDP_HIP(hipStreamSynchronize(pl->stream));
+    if (aborted) {
+        // Not every block of the fused launch was resident (the device is shared) or a wait ran out:
+        // nothing of that run is kept; do the same work with one launch per layer instead.
+        pl->ran = false;
+        pl->fused = false;
+        pl->fused_gave_up = true;
+        if (pl->no_fallback)
+            return fail(GDP_E_HIP, "fused launch: a bounded wait ran out before its tiles were finished");
+        return run(pl, mode, t);
+    }
     pl->ran = true;
     if (t) {
         memset(t, 0, sizeof *t);
@@ -454,6 +623,37 @@ int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r)
     g_err.clear();
     if (!plan || !r) return fail(GDP_E_BADARG, "null plan or results");
     return fetch(plan, r);
+}
+
+int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
+{
+    g_err.clear();
+    if (!plan) return fail(GDP_E_BADARG, "null plan");
+    switch (option) {
+        case GDP_OPT_FUSED:
+            if (value != 0 && !plan->can_fuse)
+                return fail(GDP_E_BADARG, "plan was laid out with two cost buffers (per-layer launches only)");
+            plan->fused = value != 0;
+            return GDP_OK;
+        case GDP_OPT_POISON:
+            plan->poison = value != 0;
+            return GDP_OK;
+        case GDP_OPT_NO_FALLBACK:
+            plan->no_fallback = value != 0;
+            return GDP_OK;
+        case GDP_OPT_SPIN_LIMIT: {
+            if (value < 1) return fail(GDP_E_BADARG, "spin limit must be >= 1");
+            plan->spin_limit = value;
+            GDP_HIP(hipSetDevice(plan->device));
+            for (const Group &g : plan->groups) {  // patch the device copies
+                GdpSched *sc = reinterpret_cast<GdpSched *>(plan->dbase + g.off_sched);
+                GDP_HIP(hipMemcpy(&sc->spin_limit, &value, sizeof value, hipMemcpyHostToDevice));
+            }
+            return GDP_OK;
+        }
+        default:
+            return fail(GDP_E_BADARG, "unknown option");
+    }
 }
 
 void gdp_plan_destroy(gdp_plan *plan) { destroy(plan); }

@@ -2,40 +2,61 @@
 //
 // Layout of one instance in HBM (all per instance, one sub-allocation each):
 //
-//   H[2]   two cost buffers, each (S+1) rows of `ld` doubles, row = strategy.
-//          Row s, element P+u holds h[u][s] = min over source strategies of
-//          ((f_prev[u][s'] + inter[s'][s]) + intra[s]) for SOURCE row u, i.e. the value
-//          the reference stores at f[u + mem[l][s]][s] (csrc/dp_core.cpp:67-73).  The
-//          first P elements of every row are +inf for good, so that reading
-//          f[v][s] = H[s][P + v - mem[l][s]] yields +inf for v < mem[l][s]
-//          (csrc/dp_core.cpp:60-64) without a branch.  Row S is +inf everywhere and
-//          stands in for strategies whose mem reaches V.
-//   M      argmin table, L*S rows of `ldm` entries (one byte each), indexed by the
-//          SOURCE row u like H: mark[l][v][s] of the reference is M[l][s][v - mem[l][s]].
-//   roff   (L+1) rows of S+1 int64: element offset, from the base of a cost buffer, at
-//          which "f of the previous layer, strategy s', row 0" is found.
-//   inter  n_inter matrices, each S+1 rows (last row zero) of SP doubles (columns
-//          padded with zeros up to SP = a multiple of the target tile).
+//   H      nbuf cost buffers of (S+1) rows of `ld` doubles each, row = strategy; layer l reads
+//          buffer l % nbuf and writes buffer (l+1) % nbuf.  nbuf is L+1 when all layers run in one
+//          launch (no address is ever rewritten inside that launch, so a cache line read by some
+//          XCD can never be a stale copy) and 2 when every layer is its own launch.
+//          Row s, element P+u holds
+//          h[u][s] = min over source strategies of ((f_prev[u][s'] + inter[s'][s]) + intra[s])
+//          for SOURCE row u, i.e. the value the reference stores at f[u + mem[l][s]][s]
+//          (csrc/dp_core.cpp:67-73).  The first P elements of every row are +inf for good, so
+//          that reading f[v][s] = H[s][P + v - mem[l][s]] yields +inf for v < mem[l][s]
+//          (csrc/dp_core.cpp:60-64) without a branch.  Row S is +inf everywhere and stands in
+//          for strategies whose mem reaches V and for the padding source strategies.
+//   M      argmin table, L*S rows of `ldm` entries (one byte each), indexed by the SOURCE row u
+//          like H: mark[l][v][s] of the reference is M[l][s][v - mem[l][s]].
+//   roff   (L+1) rows of SU+1 int64: element offset, from the base of a cost buffer, at which
+//          "f of the previous layer, strategy s', row 0" is found (SU = S rounded up to the
+//          source unroll; the padding entries point at the +inf row).
+//   inter  n_inter matrices, each SU+1 rows (rows >= S zero) of SP doubles (columns padded with
+//          zeros up to SP = a multiple of the target tile).
 //   intra  L rows of SP doubles (zero padded).
 //   mem    L rows of S int32, as given.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#define GDP_WAVES_PER_BLOCK 4
+#define GDP_SRC_UNROLL 2  // source strategies are consumed in groups of this many
+#define GDP_QUEUES 64     // ticket sub-queues per layer of a fused launch
+
 struct GdpDevInst {
-    double *H[2];
+    double *H;        // buffer b starts at H + b * hstride
+    int64_t hstride;  // (S+1) * ld
     uint8_t *M;
     const double *inter;
     const double *intra;
     const int32_t *inter_index;
     const int64_t *roff;
     const int32_t *mem;
-    int64_t ld;   // elements per row of H
-    int64_t ldm;  // entries per row of M
+    const int32_t *dep;  // [L] tiles below a tile that a reader of layer l's output needs
+    int64_t ld;          // elements per row of H
+    int64_t ldm;         // entries per row of M
     int32_t L, V, S, SP;
+    int32_t SU;     // S rounded up to GDP_SRC_UNROLL
     int32_t P;      // +inf elements in front of every H row
-    int32_t ntile;  // row tiles of GDP_TILE_ROWS rows covering [0, V)
-    int32_t pad0, pad1;
+    int32_t ntile;  // row tiles covering [0, V)
+    int32_t nbuf;
+};
+
+// Bookkeeping of one fused (all layers) launch over a group of instances.
+struct GdpSched {
+    int32_t *next;            // [max_L][GDP_QUEUES] ticket counters                (zeroed per run)
+    int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
+    int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
+    const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
+    int32_t max_L, max_ntile, ntb, nbt;  // nbt = block tasks per instance and layer
+    int64_t spin_limit;       // polls before a waiting wave gives up
 };
 
 struct GdpDevKey {
@@ -51,17 +72,32 @@ struct GdpDevOut {
     int32_t feasible;
 };
 
-// rows of the budget axis handled by one wavefront (64 lanes x GDP_R rows per lane)
-#define GDP_TS 8
-#define GDP_R 4
-#define GDP_TILE_ROWS (64 * GDP_R)
-#define GDP_WAVES_PER_BLOCK 4
+// Register tile of the relaxation kernel: TS target strategies x (64 lanes x R rows) per wavefront.
+struct GdpVariant {
+    int ts, r;
+};
+static const GdpVariant GDP_VARIANTS[] = {{8, 4}, {8, 2}, {8, 1}, {11, 3}, {11, 2}, {11, 1}};
+#define GDP_NUM_VARIANTS 6
 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
-hipError_t gdp_launch_relax(const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
+hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
                             hipStream_t stream);
-// Sets up H: +inf pads and +inf row in both buffers, zeros in the data region of buffer 0.
-hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, hipStream_t stream);
+// All layers of a group in one launch: blocks draw (layer, instance, tile) tasks from ticket
+// counters and wait on per-tile completion counters instead of on a kernel boundary.
+hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
+                                  hipStream_t stream);
+// Resident blocks per CU of the fused kernel (for sizing its grid).
+hipError_t gdp_fused_blocks_per_cu(int variant, int *blocks);
+// Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
+// GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
+// in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).
+#define GDP_INIT_PADS 1
+#define GDP_INIT_ZERO 2
+#define GDP_INIT_POISON 4
+hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, int max_nbuf, int what,
+                           hipStream_t stream);
+// Fills n int32 with zero (queue counters; a kernel rather than a memset so that it can be captured).
+hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream);
 // argmin over the last layer's row + backtrack, one wavefront per key.
 hipError_t gdp_launch_epilogue(const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,
                                int32_t *res, hipStream_t stream);

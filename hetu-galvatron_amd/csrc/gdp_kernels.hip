@@ -39,32 +39,29 @@ __device__ __forceinline__ unsigned xcd_swizzle(unsigned x, unsigned nblk)
     return (x & 7u) * (nblk >> 3) + (x >> 3);
 }
 
-template <int TS, int R>
-__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
-    const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
+// One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of layer `layer`.
+// PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
+// waits for this task's completion counter finds them in memory.
+template <int TS, int R, bool PUBLISH>
+__device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb,
+                                           unsigned lane)
 {
-    const GdpDevInst *I = insts + blockIdx.y;
-    const int L = uload(&I->L);
-    if (layer >= L) return;
-    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned lane = threadIdx.x & 63u;
-    const unsigned task = xcd_swizzle(blockIdx.x, nblk_x) * GDP_WAVES_PER_BLOCK + wave;
-    const unsigned tile = task / ntb;
-    const unsigned tb = task - tile * ntb;
-    if (tile >= (unsigned)uload(&I->ntile)) return;
-
     const int S = uload(&I->S);
+    const int SU = uload(&I->SU);
     const int SP = uload(&I->SP);
     const int P = uload(&I->P);
     const int64_t ld = uload(&I->ld);
     const int64_t ldm = uload(&I->ldm);
-    const double *src = uload(&I->H[layer & 1]);
-    double *dst = uload(&I->H[(layer + 1) & 1]);
+    const int nbuf = uload(&I->nbuf);
+    const int64_t hstride = uload(&I->hstride);
+    double *const hbase = uload(&I->H);
+    const double *src = hbase + (int64_t)(layer % nbuf) * hstride;
+    double *dst = hbase + (int64_t)((layer + 1) % nbuf) * hstride;
     uint8_t *M = uload(&I->M);
-    const int64_t *ro = uload(&I->roff) + (int64_t)layer * (S + 1);
+    const int64_t *ro = uload(&I->roff) + (int64_t)layer * (SU + GDP_SRC_UNROLL);
     const int s0 = tb * TS;
     const int mat = uload(uload(&I->inter_index) + layer);
-    const double *it = uload(&I->inter) + (int64_t)mat * (S + 1) * SP + s0;
+    const double *it = uload(&I->inter) + (int64_t)mat * (SU + GDP_SRC_UNROLL) * SP + s0;
     const double *ia = uload(&I->intra) + (int64_t)layer * SP + s0;
     const int64_t u0 = (int64_t)tile * (64 * R);
 
@@ -82,37 +79,56 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
             arg[r][j] = 0;
         }
 
-    double fp[R], sc[TS];
+    // Two register sets (A: even source strategies, B: odd) so that the loads for strategy sp+2 are
+    // in flight while strategy sp+1 is being consumed.  Entries SU, SU+1 of roff / inter are valid
+    // dummies, and source strategies in [S, SU) read the +inf row: +inf never wins a strict '<'.
+    double fpA[R], fpB[R], scA[TS], scB[TS];
     {
-        const double *p = src + uload(ro) + u0;
+        const double *pa = src + uload(ro) + u0;
+        const double *pb = src + uload(ro + 1) + u0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) fp[r] = p[lane + 64u * r];
+        for (int r = 0; r < R; ++r) fpA[r] = pa[lane + 64u * r];
 #pragma unroll
-        for (int j = 0; j < TS; ++j) sc[j] = uload(it + j);
+        for (int r = 0; r < R; ++r) fpB[r] = pb[lane + 64u * r];
+#pragma unroll
+        for (int j = 0; j < TS; ++j) scA[j] = uload(it + j);
+#pragma unroll
+        for (int j = 0; j < TS; ++j) scB[j] = uload(it + SP + j);
     }
 
-    for (int sp = 0; sp < S; ++sp) {
-        // prefetch the next source strategy (row S of roff / inter is a valid dummy)
-        double fpn[R], scn[TS];
-        const double *pn = src + uload(ro + sp + 1) + u0;
-#pragma unroll
-        for (int r = 0; r < R; ++r) fpn[r] = pn[lane + 64u * r];
-#pragma unroll
-        for (int j = 0; j < TS; ++j) scn[j] = uload(it + (int64_t)(sp + 1) * SP + j);
-
+    for (int sp = 0; sp < SU; sp += 2) {
 #pragma unroll
         for (int j = 0; j < TS; ++j)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const double c = (fp[r] + sc[j]) + add[j];
+                const double c = (fpA[r] + scA[j]) + add[j];
                 const bool lt = c < best[r][j];
                 best[r][j] = min_f64(best[r][j], c);
                 arg[r][j] = lt ? sp : arg[r][j];
             }
+        {
+            const double *pn = src + uload(ro + sp + 2) + u0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) fp[r] = fpn[r];
+            for (int r = 0; r < R; ++r) fpA[r] = pn[lane + 64u * r];
 #pragma unroll
-        for (int j = 0; j < TS; ++j) sc[j] = scn[j];
+            for (int j = 0; j < TS; ++j) scA[j] = uload(it + (int64_t)(sp + 2) * SP + j);
+        }
+#pragma unroll
+        for (int j = 0; j < TS; ++j)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const double c = (fpB[r] + scB[j]) + add[j];
+                const bool lt = c < best[r][j];
+                best[r][j] = min_f64(best[r][j], c);
+                arg[r][j] = lt ? (sp + 1) : arg[r][j];
+            }
+        {
+            const double *pn = src + uload(ro + sp + 3) + u0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) fpB[r] = pn[lane + 64u * r];
+#pragma unroll
+            for (int j = 0; j < TS; ++j) scB[j] = uload(it + (int64_t)(sp + 3) * SP + j);
+        }
     }
 
 #pragma unroll
@@ -123,16 +139,180 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
             uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                drow[lane + 64u * r] = best[r][j];
+                if (PUBLISH)
+                    __hip_atomic_store(drow + (lane + 64u * r), best[r][j], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    drow[lane + 64u * r] = best[r][j];
                 mrow[lane + 64u * r] = (uint8_t)arg[r][j];
             }
         }
     }
 }
 
-// +inf pads / +inf row in both buffers, zeros in the data region of buffer 0
-// (the caller's f is all zeros on entry: dynamic_programming.py:16).
-__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts)
+// ---- one launch per layer ------------------------------------------------------------------------
+template <int TS, int R>
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
+    const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
+{
+    const GdpDevInst *I = insts + blockIdx.y;
+    if (layer >= uload(&I->L)) return;
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned task = xcd_swizzle(blockIdx.x, nblk_x) * GDP_WAVES_PER_BLOCK + wave;
+    const unsigned tile = task / ntb;
+    const unsigned tb = task - tile * ntb;
+    if (tile >= (unsigned)uload(&I->ntile)) return;
+    relax_task<TS, R, false>(I, layer, tile, tb, lane);
+}
+
+// ---- all layers in one launch --------------------------------------------------------------------
+// Agent-scope (all XCDs) relaxed load / add of a queue word.
+__device__ __forceinline__ int ld_agent(const int32_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Waits until cnt[lo..hi] have all reached `full`.  The first poll comes at once; after a miss the
+// wave sleeps, longer each time (all waiting waves of a layer look at the same few cache lines, and
+// polling them back to back would queue the very counter updates they are waiting for behind the
+// polls).  Every wait is bounded: after `limit` polls, or as soon as another wave has given up, the
+// wave gives up too (returns false) and the launch drains.
+__device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, int full, unsigned lane,
+                                           int32_t *abort_flag, int64_t limit)
+{
+    int64_t polls = 0;
+    for (int base = lo; base <= hi; base += 64) {
+        const int t = base + (int)lane;
+        for (;;) {
+            const int v = (t <= hi) ? ld_agent(cnt + t) : full;
+            if (__builtin_amdgcn_ballot_w64(v < full) == 0) break;  // wave-uniform
+            ++polls;
+            const int stop = (polls & 15) ? 0 : __builtin_amdgcn_readfirstlane(ld_agent(abort_flag));
+            if (polls > limit || stop != 0) {
+                if (lane == 0) __hip_atomic_store(abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return false;
+            }
+            if (polls < 4) __builtin_amdgcn_s_sleep(32);        // ~1 us
+            else __builtin_amdgcn_s_sleep(127);                  // ~3.5 us
+        }
+    }
+    return true;
+}
+
+// Blocks draw block tasks (four consecutive (tile, target block) wave tasks of one instance and
+// layer) from ticket counters, layer by layer: all tickets of layer l are handed out before any of
+// layer l+1.  Whatever a task waits for therefore was handed out earlier and is running or
+// finished, the oldest unfinished task never waits, and the launch cannot deadlock whatever the
+// residency of its blocks.  Drawing tickets (rather than owning a fixed share) also keeps the four
+// waves of a SIMD out of step with each other, so that one wave's loads, stores and waits are
+// covered by the arithmetic of the others.
+//
+// Instead of a kernel boundary between layers, a task waits only for the tiles it reads: layer l,
+// tile t reads rows of layer l-1's output in tiles [t-dep[l-1], t].  Every layer has its own cost
+// buffer inside a fused launch, so nothing is overwritten and read-after-write is the only
+// dependence.
+//
+// Visibility across the 8 XCDs, whose L2s are not coherent with each other:
+//  - a cost cell is written once per launch with a write-through (agent scope) store, the writer
+//    waits for its stores to be acknowledged and only then bumps its tile's counter;
+//  - a reader polls the counter with agent-scope loads and only afterwards touches the tile.  Its
+//    L2 cannot hold an older copy of those lines: tiles are whole cache lines, nobody reads a tile
+//    before its counter is full, and the caches are invalidated when the launch begins.
+//
+// The tickets of a layer are dealt round-robin to GDP_QUEUES sub-queues and a block always draws
+// from sub-queue blockIdx % GDP_QUEUES, so that no single counter is hit by every block (a
+// same-address atomic is serialised at the memory side).  Each sub-queue is handed out layer by
+// layer, which is all the no-deadlock argument needs as long as one block per sub-queue runs.
+template <int TS, int R>
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
+    const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q)
+{
+    __shared__ int sh_ticket[2];
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned lane = threadIdx.x & 63u;
+    const int max_L = uload(&Q->max_L);
+    const int max_ntile = uload(&Q->max_ntile);
+    const int ntb = uload(&Q->ntb);
+    const int nbt = uload(&Q->nbt);
+    int32_t *next = uload(&Q->next);
+    int32_t *cnt_all = uload(&Q->cnt);
+    int32_t *abort_flag = uload(&Q->abort_flag);
+    const int32_t *n_active = uload(&Q->n_active);
+    const int64_t limit = uload(&Q->spin_limit);
+    const int qid = (int)(blockIdx.x % GDP_QUEUES);
+    int layer = 0;
+    for (;;) {
+        // ---- wave 0 draws the next ticket and waits for what the block's four wave tasks read -----
+        if (wave == 0) {
+            int ticket = -1;
+            while (layer < max_L) {
+                const int total = uload(n_active + layer) * nbt;
+                int k = 0;
+                if (lane == 0)
+                    k = __hip_atomic_fetch_add(next + layer * GDP_QUEUES + qid, 1, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                k = __builtin_amdgcn_readfirstlane(k);
+                ticket = k * GDP_QUEUES + qid;
+                if (ticket < total) break;
+                ticket = -1;
+                ++layer;
+            }
+            if (ticket >= 0 && layer >= 1) {
+                const int nat = uload(n_active + layer);
+                const int bt = ticket / nat;
+                const int ii = ticket - bt * nat;
+                const GdpDevInst *I = insts + ii;
+                const int ntile = uload(&I->ntile);
+                const unsigned q0 = (unsigned)bt * GDP_WAVES_PER_BLOCK;
+                const int t_lo = (int)(q0 / (unsigned)ntb);
+                int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / (unsigned)ntb);
+                if (t_hi >= ntile) t_hi = ntile - 1;
+                if (t_lo < ntile) {
+                    const int d = uload(uload(&I->dep) + layer - 1);
+                    const int lo = t_lo - d < 0 ? 0 : t_lo - d;
+                    const int32_t *cnt_prev =
+                        cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile;
+                    if (!wait_tiles(cnt_prev, lo, t_hi, ntb, lane, abort_flag, limit)) ticket = -1;
+                }
+            }
+            if (ticket >= 0 && __builtin_amdgcn_readfirstlane(ld_agent(abort_flag)) != 0) ticket = -1;
+            if (lane == 0) {
+                sh_ticket[0] = ticket;
+                sh_ticket[1] = layer;
+            }
+        }
+        __syncthreads();
+        const int ticket = __builtin_amdgcn_readfirstlane(sh_ticket[0]);
+        layer = __builtin_amdgcn_readfirstlane(sh_ticket[1]);
+        __syncthreads();  // sh_ticket is rewritten only after every wave has read it
+        if (ticket < 0) return;  // out of work, or the launch is being abandoned (block-uniform)
+        const int nat = uload(n_active + layer);
+        const int bt = ticket / nat;       // block task within the instance: tiles ascend with tickets
+        const int ii = ticket - bt * nat;  // instance (a prefix of the table is active)
+        const GdpDevInst *I = insts + ii;
+        const unsigned q = (unsigned)bt * GDP_WAVES_PER_BLOCK + wave;
+        const unsigned tile = q / (unsigned)ntb;
+        const unsigned tb = q - tile * (unsigned)ntb;
+        if (tile >= (unsigned)uload(&I->ntile)) continue;  // wave-uniform; the barriers are per ticket
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the tile's loads after the wait
+        relax_task<TS, R, true>(I, layer, tile, tb, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every write-through store acknowledged
+        if (lane == 0)
+            __hip_atomic_fetch_add(cnt_all + ((int64_t)ii * max_L + layer) * max_ntile + tile, 1, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+__global__ __launch_bounds__(256) void gdp_zero_kernel(int32_t *p, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = 0;
+}
+
+// Fills of the cost buffers (see GDP_INIT_* in gdp_kernels.h).  grid = (x chunks, rows 0..S, instances).
+__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts, int what)
 {
     const GdpDevInst *I = insts + blockIdx.z;
     const int S = uload(&I->S);
@@ -140,13 +320,21 @@ __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restr
     if (row > S) return;
     const int64_t ld = uload(&I->ld);
     const int P = uload(&I->P);
-    double *h0 = uload(&I->H[0]) + (int64_t)row * ld;
-    double *h1 = uload(&I->H[1]) + (int64_t)row * ld;
+    const int nbuf = uload(&I->nbuf);
+    const int64_t hstride = uload(&I->hstride);
+    double *h = uload(&I->H) + (int64_t)row * ld;
     const double inf = INFINITY;
+    const double nan = __builtin_nan("");
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ld; i += (int64_t)gridDim.x * blockDim.x) {
         const bool pad = (row == S) || (i < P);
-        h0[i] = pad ? inf : 0.0;
-        if (pad) h1[i] = inf;
+        if (pad) {
+            if (what & GDP_INIT_PADS)
+                for (int b = 0; b < nbuf; ++b) h[(int64_t)b * hstride + i] = inf;
+        } else {
+            if (what & GDP_INIT_ZERO) h[i] = 0.0;
+            if (what & GDP_INIT_POISON)
+                for (int b = 1; b < nbuf; ++b) h[(int64_t)b * hstride + i] = nan;
+        }
     }
 }
 
@@ -211,8 +399,8 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
         if (lane == 0) out[blockIdx.x] = o;
         return;
     }
-    const double *fin = uload(&I->H[L & 1]);  // layer l writes buffer (l+1)&1
-    const int64_t *ro = uload(&I->roff) + (int64_t)L * (S + 1);
+    const double *fin = uload(&I->H) + (int64_t)(L % uload(&I->nbuf)) * uload(&I->hstride);  // last written
+    const int64_t *ro = uload(&I->roff) + (int64_t)L * (uload(&I->SU) + GDP_SRC_UNROLL);
     double val = INFINITY;
     int idx = 0x7fffffff;
     for (int s = lane; s < S; s += 64) {  // ascending within the lane: strict '<' keeps the first
@@ -235,8 +423,15 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
     for (int i = L - 1; i > 0; --i) {  // csrc/dp_core.cpp:105-113, with mark[i][v][s] = M[i][s][v - mem[i][s]]
         const int cur = idx;
         v -= mem[(int64_t)i * S + cur];
+        if (v < 0) break;  // cannot happen on a finite path; keeps a damaged table from being indexed
         idx = M[((int64_t)i * S + cur) * ldm + v];
+        if (idx >= S) { v = -1; break; }
         path[i - 1] = idx;
+    }
+    if (v < 0) {
+        o.total = INFINITY;
+        out[blockIdx.x] = o;
+        return;
     }
     o.remaining = (int32_t)(v - mem[idx]);  // csrc/dp_core.cpp:115
     o.feasible = 1;
@@ -247,8 +442,8 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
 __global__ __launch_bounds__(256) void gdp_export_f_kernel(const GdpDevInst *__restrict__ I, double *__restrict__ f)
 {
     const int L = I->L, V = I->V, S = I->S;
-    const double *fin = I->H[L & 1];
-    const int64_t *ro = I->roff + (int64_t)L * (S + 1);
+    const double *fin = I->H + (int64_t)(L % I->nbuf) * I->hstride;
+    const int64_t *ro = I->roff + (int64_t)L * (I->SU + GDP_SRC_UNROLL);
     const int64_t n = (int64_t)V * S;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t v = i / S;
@@ -275,24 +470,87 @@ __global__ __launch_bounds__(256) void gdp_export_mark_kernel(const GdpDevInst *
 
 }  // namespace
 
-hipError_t gdp_launch_relax(const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
-                            hipStream_t stream)
+template <int TS, int R>
+static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_ntile_rows, int SP, int layer,
+                                 hipStream_t stream)
 {
-    const unsigned ntb = (unsigned)(SP / GDP_TS);
-    const unsigned tasks = (unsigned)max_ntile * ntb;
+    const unsigned ntb = (unsigned)(SP / TS);
+    const unsigned tasks = (unsigned)max_ntile_rows * ntb;
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     nblk = (nblk + 7u) & ~7u;
     dim3 grid(nblk, (unsigned)n_inst, 1), block(64 * GDP_WAVES_PER_BLOCK, 1, 1);
-    hipLaunchKernelGGL((gdp_relax_kernel<GDP_TS, GDP_R>), grid, block, 0, stream, insts, layer, ntb, nblk);
+    hipLaunchKernelGGL((gdp_relax_kernel<TS, R>), grid, block, 0, stream, insts, layer, ntb, nblk);
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, hipStream_t stream)
+hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
+                            hipStream_t stream)
 {
+    switch (variant) {
+        case 0: return launch_relax_t<8, 4>(insts, n_inst, max_ntile, SP, layer, stream);
+        case 1: return launch_relax_t<8, 2>(insts, n_inst, max_ntile, SP, layer, stream);
+        case 2: return launch_relax_t<8, 1>(insts, n_inst, max_ntile, SP, layer, stream);
+        case 3: return launch_relax_t<11, 3>(insts, n_inst, max_ntile, SP, layer, stream);
+        case 4: return launch_relax_t<11, 2>(insts, n_inst, max_ntile, SP, layer, stream);
+        case 5: return launch_relax_t<11, 1>(insts, n_inst, max_ntile, SP, layer, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
+                                  hipStream_t stream)
+{
+    dim3 grid((unsigned)grid_blocks), block(64 * GDP_WAVES_PER_BLOCK);
+#define GDP_FUSED_CASE(id, ts, r) \
+    case id: hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r>), grid, block, 0, stream, insts, sched); break;
+    switch (variant) {
+        GDP_FUSED_CASE(0, 8, 4)
+        GDP_FUSED_CASE(1, 8, 2)
+        GDP_FUSED_CASE(2, 8, 1)
+        GDP_FUSED_CASE(3, 11, 3)
+        GDP_FUSED_CASE(4, 11, 2)
+        GDP_FUSED_CASE(5, 11, 1)
+        default: return hipErrorInvalidValue;
+    }
+#undef GDP_FUSED_CASE
+    return hipGetLastError();
+}
+
+hipError_t gdp_fused_blocks_per_cu(int variant, int *blocks)
+{
+#define GDP_OCC_CASE(id, ts, r)                                                                      \
+    case id:                                                                                         \
+        return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks, gdp_relax_fused_kernel<ts, r>, \
+                                                            64 * GDP_WAVES_PER_BLOCK, 0);
+    switch (variant) {
+        GDP_OCC_CASE(0, 8, 4)
+        GDP_OCC_CASE(1, 8, 2)
+        GDP_OCC_CASE(2, 8, 1)
+        GDP_OCC_CASE(3, 11, 3)
+        GDP_OCC_CASE(4, 11, 2)
+        GDP_OCC_CASE(5, 11, 1)
+        default: return hipErrorInvalidValue;
+    }
+#undef GDP_OCC_CASE
+}
+
+hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    unsigned nb = (unsigned)((n + 1023) / 1024);
+    if (nb > 4096u) nb = 4096u;
+    hipLaunchKernelGGL(gdp_zero_kernel, dim3(nb), dim3(256), 0, stream, p, n);
+    return hipGetLastError();
+}
+
+hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, int max_nbuf, int what,
+                           hipStream_t stream)
+{
+    (void)max_nbuf;
     unsigned bx = (unsigned)((max_ld + 256 * 8 - 1) / (256 * 8));
     if (bx == 0) bx = 1;
     dim3 grid(bx, (unsigned)(max_S + 1), (unsigned)n_inst), block(256, 1, 1);
-    hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts);
+    hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts, what);
     return hipGetLastError();
 }
 

@@ -21,19 +21,19 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-shared"
                "-Wno-unused-command-line-argument"]
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
+def build(verbose: bool = False, extra_flags=(), out: str = LIB_PATH, csrc: str = CSRC) -> str:
+    os.makedirs(os.path.dirname(out), exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB_PATH]
+    cmd = [hipcc] + HIPCC_FLAGS + list(extra_flags) + [os.path.join(csrc, s) for s in SOURCES] + ["-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+    log = "\n".join(l for l in proc.stdout.splitlines() if "is not a recognized feature for this target" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
-    return LIB_PATH
+        raise RuntimeError("hipcc failed:\n" + log)
+    if verbose and log.strip():
+        print(log)
+    return out
 
 
 if __name__ == "__main__":

@@ -12,7 +12,8 @@ from typing import Sequence
 import numpy as np
 
 PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(PKG, "lib", "libgalvatron_dp_hip.so")
+# GALVATRON_DP_HIP_LIB points at another build of the same library (e.g. a tuning variant).
+LIB_PATH = os.environ.get("GALVATRON_DP_HIP_LIB") or os.path.join(PKG, "lib", "libgalvatron_dp_hip.so")
 
 GDP_OK = 0
 GDP_E_BADARG = -1
@@ -23,9 +24,13 @@ GDP_E_HIP = -5
 GDP_EXPORT_F = 1
 GDP_EXPORT_MARK = 2
 GDP_MAX_S = 256
+GDP_OPT_FUSED = 1
+GDP_OPT_SPIN_LIMIT = 2
+GDP_OPT_POISON = 3
+GDP_OPT_NO_FALLBACK = 4
 
 EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
-                    "gdp_plan_destroy", "gdp_last_error", "gdp_version", "gdp_device_info")
+                    "gdp_plan_destroy", "gdp_plan_set_option", "gdp_last_error", "gdp_version", "gdp_device_info")
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -74,6 +79,8 @@ def lib() -> ctypes.CDLL:
         L.gdp_plan_run.restype = ctypes.c_int
         L.gdp_plan_fetch.argtypes = [ctypes.c_void_p, rp]
         L.gdp_plan_fetch.restype = ctypes.c_int
+        L.gdp_plan_set_option.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64]
+        L.gdp_plan_set_option.restype = ctypes.c_int
         L.gdp_plan_destroy.argtypes = [ctypes.c_void_p]
         L.gdp_plan_destroy.restype = None
         L.gdp_last_error.argtypes = []
@@ -184,6 +191,9 @@ class Plan:
         h = ctypes.c_void_p()
         _check(lib().gdp_plan_create(len(self.problems), self._P, ctypes.byref(h)))
         self._h = h
+
+    def set_option(self, option: int, value: int) -> None:
+        _check(lib().gdp_plan_set_option(self._h, option, value))
 
     def run(self, timing_mode: int = 0) -> gdp_timing:
         t = gdp_timing()

@@ -110,6 +110,22 @@ int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing);
 int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r);
 void gdp_plan_destroy(gdp_plan *plan);
 
+/* Tuning / test knobs of a plan (no counterpart in the reference).
+ *   GDP_OPT_FUSED      1 (default): all layers run in ONE launch, every block owns a fixed share of
+ *                      the (layer, instance, tile) tasks and waits on per-tile counters;
+ *                      0: one launch per layer.  Results are identical.  A plan created with
+ *                      GALVATRON_DP_FUSED=0 in the environment, or whose per-layer cost buffers
+ *                      did not fit in device memory, keeps two cost buffers and cannot be
+ *                      switched to 1.
+ *   GDP_OPT_SPIN_LIMIT polls a waiting wavefront makes before it gives up; when that happens the
+ *                      launch drains normally, the plan switches itself to one launch per layer
+ *                      and the run is repeated that way (GDP_E_HIP with GDP_OPT_NO_FALLBACK). */
+#define GDP_OPT_FUSED 1
+#define GDP_OPT_SPIN_LIMIT 2
+#define GDP_OPT_POISON 3 /* test aid: NaN-fill every not-yet-written cost buffer before each run */
+#define GDP_OPT_NO_FALLBACK 4 /* test aid: an abandoned fused launch is an error, not a switch to per-layer */
+int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
+
 /* Text of the calling thread's last error ("" if none). */
 const char *gdp_last_error(void);
 /* GDP_VERSION of the built library. */
