@@ -183,7 +183,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     pl->n = n;
     GDP_HIP(hipGetDevice(&pl->device));
     // defaults of the plan options can be preset from the environment
-    if (const char *e = getenv("GALVATRON_DP_FUSED")) pl->fused = atoi(e) != 0;
+    bool fused_preset = false;
+    if (const char *e = getenv("GALVATRON_DP_FUSED")) {
+        pl->fused = atoi(e) != 0;
+        fused_preset = true;
+    }
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_SPIN_LIMIT")) {
@@ -242,6 +246,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         }
         if (pl->tile_r_override > 0 && find_variant(ts, pl->tile_r_override) >= 0) best_r = pl->tile_r_override;
         g.variant = find_variant(ts, best_r);
+        if (g.variant < 0) return fail(GDP_E_BADARG, "no kernel variant for the requested tile/scan override");
         const int tile_rows = 64 * best_r;
         g.SP = ntb * ts;
         g.ntb = ntb;
@@ -264,6 +269,19 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         pl->max_L = std::max(pl->max_L, g.max_L);
         pl->groups.push_back(g);
         i = j;
+    }
+    for (int i = 0; i < n && !fused_preset; ++i) {  // an explicit request of the caller
+        if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
+        else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
+    }
+    if (!fused_preset) {
+        // One launch for all layers pays off when a layer holds several times more block tasks than
+        // the device holds blocks: then the tasks a block waits for were finished long before, and
+        // its loads, stores and waits hide under the arithmetic of its neighbours.  A layer that
+        // barely fills the device is better off with a launch of its own.
+        int64_t first_layer = 0;
+        for (const Group &g : pl->groups) first_layer += (int64_t)g.active[0] * g.nbt;
+        pl->fused = first_layer >= 4 * (int64_t)pl->num_cu * 4;
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -299,7 +317,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     pl->off_zero = off;
     pl->off_abort = take(sizeof(int32_t));
     for (auto &g : pl->groups) {
-        g.off_next = take(sizeof(int32_t) * (size_t)g.max_L * GDP_QUEUES);
+        g.off_next = take(sizeof(int32_t) * (size_t)g.max_L);
         g.off_cnt = take(sizeof(int32_t) * (size_t)g.count * g.max_L * g.max_ntile);
     }
     pl->zero_words = (off - pl->off_zero) / sizeof(int32_t);
@@ -425,7 +443,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         int want = 4;  // resident blocks per CU (16 waves, 4 per SIMD)
         if (const char *e = getenv("GALVATRON_DP_BLOCKS_PER_CU")) want = std::max(1, atoi(e));
         int64_t grid = std::min<int64_t>(first_layer, (int64_t)std::max(std::min(per_cu, want), 1) * pl->num_cu);
-        g.grid_blocks = (int)std::max<int64_t>(GDP_QUEUES, grid / GDP_QUEUES * GDP_QUEUES);
+        g.grid_blocks = (int)std::max<int64_t>(1, grid);
         (void)tasks;
     }
     GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));

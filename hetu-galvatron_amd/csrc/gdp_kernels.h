@@ -15,11 +15,12 @@
 //          for strategies whose mem reaches V and for the padding source strategies.
 //   M      argmin table, L*S rows of `ldm` entries (one byte each), indexed by the SOURCE row u
 //          like H: mark[l][v][s] of the reference is M[l][s][v - mem[l][s]].
-//   roff   (L+1) rows of SU+1 int64: element offset, from the base of a cost buffer, at which
-//          "f of the previous layer, strategy s', row 0" is found (SU = S rounded up to the
-//          source unroll; the padding entries point at the +inf row).
-//   inter  n_inter matrices, each SU+1 rows (rows >= S zero) of SP doubles (columns padded with
-//          zeros up to SP = a multiple of the target tile).
+//   roff   (L+1) rows of SU+GDP_SRC_UNROLL int64: element offset, from the base of a cost buffer,
+//          at which "f of the previous layer, strategy s', row 0" is found (SU = S rounded up to
+//          the source unroll; the entries from S on point at the +inf row: padding sources and the
+//          targets of the last prefetches).
+//   inter  n_inter matrices, each SU+GDP_SRC_UNROLL rows (rows >= S zero) of SP doubles (columns
+//          padded with zeros up to SP = a multiple of the target tile).
 //   intra  L rows of SP doubles (zero padded).
 //   mem    L rows of S int32, as given.
 #pragma once
@@ -27,8 +28,7 @@
 #include <stdint.h>
 
 #define GDP_WAVES_PER_BLOCK 4
-#define GDP_SRC_UNROLL 2  // source strategies are consumed in groups of this many
-#define GDP_QUEUES 64     // ticket sub-queues per layer of a fused launch
+#define GDP_SRC_UNROLL 2  // source strategies are consumed two at a time (padded with +inf sources)
 
 struct GdpDevInst {
     double *H;        // buffer b starts at H + b * hstride
@@ -51,7 +51,7 @@ struct GdpDevInst {
 
 // Bookkeeping of one fused (all layers) launch over a group of instances.
 struct GdpSched {
-    int32_t *next;            // [max_L][GDP_QUEUES] ticket counters                (zeroed per run)
+    int32_t *next;            // [max_L] ticket counter per layer                  (zeroed per run)
     int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
@@ -73,6 +73,7 @@ struct GdpDevOut {
 };
 
 // Register tile of the relaxation kernel: TS target strategies x (64 lanes x R rows) per wavefront.
+// Variants of one width are listed tallest first.
 struct GdpVariant {
     int ts, r;
 };

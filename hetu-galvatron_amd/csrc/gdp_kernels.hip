@@ -96,7 +96,8 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
         for (int j = 0; j < TS; ++j) scB[j] = uload(it + SP + j);
     }
 
-    for (int sp = 0; sp < SU; sp += 2) {
+    const int S2 = (S + 1) & ~1;
+    for (int sp = 0; sp < S2; sp += 2) {
 #pragma unroll
         for (int j = 0; j < TS; ++j)
 #pragma unroll
@@ -151,8 +152,10 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
 }
 
 // ---- one launch per layer ------------------------------------------------------------------------
+// __launch_bounds__(256, 4): register allocation is held to 4 resident blocks per CU (4 waves per
+// SIMD, at most 128 VGPRs).
 template <int TS, int R>
-__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_kernel(
     const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
 {
     const GdpDevInst *I = insts + blockIdx.y;
@@ -219,13 +222,8 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //  - a reader polls the counter with agent-scope loads and only afterwards touches the tile.  Its
 //    L2 cannot hold an older copy of those lines: tiles are whole cache lines, nobody reads a tile
 //    before its counter is full, and the caches are invalidated when the launch begins.
-//
-// The tickets of a layer are dealt round-robin to GDP_QUEUES sub-queues and a block always draws
-// from sub-queue blockIdx % GDP_QUEUES, so that no single counter is hit by every block (a
-// same-address atomic is serialised at the memory side).  Each sub-queue is handed out layer by
-// layer, which is all the no-deadlock argument needs as long as one block per sub-queue runs.
 template <int TS, int R>
-__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_kernel(
     const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q)
 {
     __shared__ int sh_ticket[2];
@@ -240,7 +238,6 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kern
     int32_t *abort_flag = uload(&Q->abort_flag);
     const int32_t *n_active = uload(&Q->n_active);
     const int64_t limit = uload(&Q->spin_limit);
-    const int qid = (int)(blockIdx.x % GDP_QUEUES);
     int layer = 0;
     for (;;) {
         // ---- wave 0 draws the next ticket and waits for what the block's four wave tasks read -----
@@ -250,10 +247,8 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kern
                 const int total = uload(n_active + layer) * nbt;
                 int k = 0;
                 if (lane == 0)
-                    k = __hip_atomic_fetch_add(next + layer * GDP_QUEUES + qid, 1, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
-                k = __builtin_amdgcn_readfirstlane(k);
-                ticket = k * GDP_QUEUES + qid;
+                    k = __hip_atomic_fetch_add(next + layer, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ticket = __builtin_amdgcn_readfirstlane(k);
                 if (ticket < total) break;
                 ticket = -1;
                 ++layer;
@@ -483,55 +478,46 @@ static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_nt
     return hipGetLastError();
 }
 
+// one entry per element of GDP_VARIANTS, in the same order
+#define GDP_FOR_EACH_VARIANT(X) X(0, 8, 4) X(1, 8, 2) X(2, 8, 1) X(3, 11, 3) X(4, 11, 2) X(5, 11, 1)
+
 hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
                             hipStream_t stream)
 {
+#define X(id, ts, r) \
+    case id: return launch_relax_t<ts, r>(insts, n_inst, max_ntile, SP, layer, stream);
     switch (variant) {
-        case 0: return launch_relax_t<8, 4>(insts, n_inst, max_ntile, SP, layer, stream);
-        case 1: return launch_relax_t<8, 2>(insts, n_inst, max_ntile, SP, layer, stream);
-        case 2: return launch_relax_t<8, 1>(insts, n_inst, max_ntile, SP, layer, stream);
-        case 3: return launch_relax_t<11, 3>(insts, n_inst, max_ntile, SP, layer, stream);
-        case 4: return launch_relax_t<11, 2>(insts, n_inst, max_ntile, SP, layer, stream);
-        case 5: return launch_relax_t<11, 1>(insts, n_inst, max_ntile, SP, layer, stream);
+        GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
     }
+#undef X
 }
 
 hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
                                   hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks), block(64 * GDP_WAVES_PER_BLOCK);
-#define GDP_FUSED_CASE(id, ts, r) \
+#define X(id, ts, r) \
     case id: hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r>), grid, block, 0, stream, insts, sched); break;
     switch (variant) {
-        GDP_FUSED_CASE(0, 8, 4)
-        GDP_FUSED_CASE(1, 8, 2)
-        GDP_FUSED_CASE(2, 8, 1)
-        GDP_FUSED_CASE(3, 11, 3)
-        GDP_FUSED_CASE(4, 11, 2)
-        GDP_FUSED_CASE(5, 11, 1)
+        GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
     }
-#undef GDP_FUSED_CASE
+#undef X
     return hipGetLastError();
 }
 
 hipError_t gdp_fused_blocks_per_cu(int variant, int *blocks)
 {
-#define GDP_OCC_CASE(id, ts, r)                                                                      \
+#define X(id, ts, r)                                                                                 \
     case id:                                                                                         \
         return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks, gdp_relax_fused_kernel<ts, r>, \
                                                             64 * GDP_WAVES_PER_BLOCK, 0);
     switch (variant) {
-        GDP_OCC_CASE(0, 8, 4)
-        GDP_OCC_CASE(1, 8, 2)
-        GDP_OCC_CASE(2, 8, 1)
-        GDP_OCC_CASE(3, 11, 3)
-        GDP_OCC_CASE(4, 11, 2)
-        GDP_OCC_CASE(5, 11, 1)
+        GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
     }
-#undef GDP_OCC_CASE
+#undef X
 }
 
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)

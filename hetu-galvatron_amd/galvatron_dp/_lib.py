@@ -23,6 +23,8 @@ GDP_E_NOMEM = -4
 GDP_E_HIP = -5
 GDP_EXPORT_F = 1
 GDP_EXPORT_MARK = 2
+GDP_LAUNCH_FUSED = 4
+GDP_LAUNCH_PER_LAYER = 8
 GDP_MAX_S = 256
 GDP_OPT_FUSED = 1
 GDP_OPT_SPIN_LIMIT = 2
@@ -117,7 +119,7 @@ class Problem:
     dtypes/layouts the C ABI wants, plus the output arrays it will fill."""
 
     def __init__(self, mem, intra, inter, V: int, other_mem: Sequence[int], other_time: Sequence[float], *,
-                 inter_index=None, export_f: bool = False, export_mark: bool = False):
+                 inter_index=None, export_f: bool = False, export_mark: bool = False, launch: str | None = None):
         self.mem = np.ascontiguousarray(mem, dtype=np.int32)
         if self.mem.ndim != 2:
             raise ValueError("mem must be [L,S]")
@@ -142,7 +144,11 @@ class Problem:
         if self.other_mem.shape != self.other_time.shape:
             raise ValueError("other_mem and other_time must have one entry per key")
         self.n_key = int(self.other_mem.shape[0])
-        self.flags = (GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0)
+        if launch not in (None, "fused", "per_layer"):
+            raise ValueError("launch must be None, 'fused' or 'per_layer'")
+        self.flags = ((GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0) |
+                      (GDP_LAUNCH_FUSED if launch == "fused" else 0) |
+                      (GDP_LAUNCH_PER_LAYER if launch == "per_layer" else 0))
         if self.V < 1 or self.L < 1 or self.S < 1:
             raise ValueError("L, V and S must be >= 1")
         # outputs

@@ -45,6 +45,8 @@ extern "C" {
 /* gdp_problem.flags */
 #define GDP_EXPORT_F 1u    /* write result.f_out    (final f, reference layout [V][S])       */
 #define GDP_EXPORT_MARK 2u /* write result.mark_out (argmin table, reference layout [L][V][S]) */
+#define GDP_LAUNCH_FUSED 4u     /* lay the plan out for, and use, ONE launch over all layers          */
+#define GDP_LAUNCH_PER_LAYER 8u /* one launch per layer (two cost buffers); default: chosen by size    */
 
 /* One DP instance == one reference call.  Field <- reference argument (csrc/dp_core.cpp:24-35):
  *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),

@@ -1,0 +1,129 @@
+"""GPU tests of the batched entry points and of the two launch schemes (one launch per layer /
+one launch for all layers), through the C ABI."""
+import numpy as np
+import pytest
+
+import helpers as H
+from galvatron_dp import _lib, workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(inst, **kw):
+    keys = sorted(inst.other_mem)
+    return _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                        [inst.other_time[k] for k in keys], inter_index=inst.inter_index, **kw)
+
+
+def _check_against_golden(prob, rec, name):
+    keys = rec["keys"]
+    got = ({k: prob.total[i] for i, k in enumerate(keys)},
+           {k: [int(x) if prob.remaining[i] != -1 else -1 for x in prob.res[i]] for i, k in enumerate(keys)},
+           {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+    H.assert_same_results(got, H.golden_results(rec), name)
+
+
+def test_batched_sweep_256_instances_matches_reference(golden):
+    """BASELINE config 3: all 256 instances of the pp x bsz x chunks sweep in ONE gdp_solve_batch
+    call, every instance compared with the reference's result for it."""
+    insts = W.config3()
+    assert len(insts) == 256
+    probs = [_problem(i) for i in insts]
+    _lib.solve_batch(probs)
+    for n, (inst, prob) in enumerate(zip(insts, probs)):
+        rec = golden[f"cfg3_{n:03d}"]
+        assert inst.digest() == rec["input_sha256"]
+        _check_against_golden(prob, rec, f"cfg3_{n:03d}")
+
+
+def test_mixed_shapes_in_one_batch(golden):
+    """Instances with different L, S and V in one call (grouped by S internally) come back in the
+    caller's order."""
+    names = ["ties_1", "rand_2", "cfg3_smallV_0", "infeasible_3", "rand_5", "cfg3_smallV_3", "ties_6", "rand_7",
+             "cfg2_small", "rand_8", "cfg4_small", "galvatron_like"]
+    insts = [H.build_case(golden[n]) for n in names]
+    probs = [_problem(i) for i in insts]
+    _lib.solve_batch(probs)
+    for n, prob in zip(names, probs):
+        _check_against_golden(prob, golden[n], n)
+
+
+@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("name", ["cfg2_small", "cfg4_small", "galvatron_like", "ties_6", "infeasible_9"])
+def test_both_launch_schemes_give_identical_arrays(golden, name, fused):
+    rec = golden[name]
+    inst = H.build_case(rec)
+    prob = _problem(inst, export_f=True, export_mark=True, launch="fused" if fused else "per_layer")
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)       # unwritten cells read as NaN: a stale read would show
+        for _ in range(2):                             # a plan can be run again and again
+            plan.run()
+            plan.fetch()
+            _check_against_golden(prob, rec, name)
+            assert H.sha(prob.f_out) == rec["f_sha256"]
+            assert H.sha(prob.mark_out) == rec["mark_sha256"]
+
+
+def test_abandoned_fused_launch_falls_back_or_reports(golden):
+    """A spin limit of 1 makes waiting wavefronts give up at once (forced from the host; every
+    kernel still runs to completion).  With the fallback the plan switches to per-layer launches
+    and returns the right answer; without it the run reports an error.  Either way the next call
+    on a fresh plan works."""
+    rec = golden["cfg2_small"]
+    inst = H.build_case(rec)
+    prob = _problem(inst, launch="fused")
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_SPIN_LIMIT, 1)
+        plan.run()
+        plan.fetch()
+        _check_against_golden(prob, rec, "fallback")
+    prob2 = _problem(inst, launch="fused")
+    with _lib.Plan([prob2]) as plan:
+        plan.set_option(_lib.GDP_OPT_SPIN_LIMIT, 1)
+        plan.set_option(_lib.GDP_OPT_NO_FALLBACK, 1)
+        try:
+            plan.run()
+            gave_up = False
+        except RuntimeError as e:
+            gave_up = True
+            assert "bounded wait" in str(e)
+        if not gave_up:                               # every wait happened to be satisfied at its first poll
+            plan.fetch()
+            _check_against_golden(prob2, rec, "no-fallback, nothing had to wait")
+    prob3 = _problem(inst)
+    _lib.solve_batch([prob3])
+    _check_against_golden(prob3, rec, "after")
+
+
+def test_shim_batch_entry_point(golden):
+    import galvatron_dp_core as shim
+    names = ["rand_1", "ties_3", "infeasible_5"]
+    calls, want = [], []
+    for n in names:
+        inst = H.build_case(golden[n])
+        res = {k: np.full(inst.L, -1, dtype=np.int32) for k in inst.other_mem}
+        calls.append((inst.L, inst.V, inst.S, inst.mem, None, None, inst.inter, inst.intra, inst.other_mem,
+                      inst.other_time, res))
+        want.append(golden[n])
+    outs = shim.dynamic_programming_core_batch(calls)
+    for (total, rem), call, rec, n in zip(outs, calls, want, names):
+        got = (total, {k: [int(x) for x in v] for k, v in call[10].items()}, rem)
+        H.assert_same_results(got, H.golden_results(rec), n)
+
+
+def test_errors_surface_as_python_exceptions():
+    import galvatron_dp_core as shim
+    L, S, V = 2, 3, 16
+    mem = np.ones((L, S), np.int32)
+    intra = np.ones((L, S))
+    inter = np.zeros((L, S, S))
+    res = {1: np.full(L, -1, np.int32)}
+    bad = mem.copy(); bad[0, 0] = 0
+    with pytest.raises(_lib.UnsupportedInputError):
+        shim.dynamic_programming_core(L, V, S, bad, None, None, inter, intra, {1: 0}, {1: 0.0}, res)
+    nan = intra.copy(); nan[1, 1] = np.nan
+    with pytest.raises(ValueError):
+        shim.dynamic_programming_core(L, V, S, mem, None, None, inter, nan, {1: 0}, {1: 0.0}, res)
+    total, rem = shim.dynamic_programming_core(L, V, S, mem, None, None, inter, intra, {1: 0, 2: 99}, {1: 0.5, 2: 0.0},
+                                               {1: res[1], 2: np.full(L, -1, np.int32)})
+    assert total == {1: 2.5, 2: np.inf} and rem == {1: V - 1 - 2, 2: -1} and list(res[1]) == [0, 0]
