@@ -37,7 +37,10 @@ PEAK_FP64_VALU_TFLOPS = 39.3   # 78.6 TFLOP/s published (FMA = 2 ops) / 2
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the relaxation kernel measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (scaled by a copy kernel of known size); see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    "cfg2": 144.4e6,    # profiles/gdp_relax_kernel_cfg2.txt        (algorithmic 142.6e6)
+    "cfg3": 227.5e9,    # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 188.2e9; one launch per solve)
+}
 
 
 def _problems(workload: str):
@@ -55,18 +58,21 @@ def _problems(workload: str):
     return insts, probs
 
 
-def _cpu_baseline(workload: str, budget_s: float = 20.0):
+def _cpu_baseline(workload: str, budget_s: float = 15.0):
     """Reference dp_core (or the C port) on the first layers of the workload's first instance."""
     import numpy as np
     from galvatron_dp import workloads as W
     from oracle import dp_oracle as O
     inst = W.config3(n_limit=1)[0] if workload == "cfg3" else W.CONFIGS[int(workload[3:])]()
     use_ref = O.ref_available()
-    rate_guess = 4.0e8 if use_ref else 5.5e8
-    per_layer = inst.V * inst.S * inst.S
-    n_layers = int(max(1, min(inst.L, budget_s * rate_guess // per_layer)))
-    mem, intra, inter = inst.mem[:n_layers], inst.intra[:n_layers], np.ascontiguousarray(inst.inter[:n_layers])
     fn = O.ref_solve if use_ref else O.solve
+    per_layer = inst.V * inst.S * inst.S
+    # one layer first to learn this host's rate, then as many layers as fit the time budget
+    t0 = time.perf_counter()
+    fn(inst.mem[:1], inst.intra[:1], np.ascontiguousarray(inst.inter[:1]), inst.V, inst.other_mem, inst.other_time)
+    rate = per_layer / (time.perf_counter() - t0)
+    n_layers = int(max(1, min(inst.L, budget_s * rate // per_layer)))
+    mem, intra, inter = inst.mem[:n_layers], inst.intra[:n_layers], np.ascontiguousarray(inst.inter[:n_layers])
     t0 = time.perf_counter()
     fn(mem, intra, inter, inst.V, inst.other_mem, inst.other_time)
     dt = time.perf_counter() - t0
@@ -86,6 +92,9 @@ def main() -> int:
     ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--also", default="cfg3", help="comma-separated extra workloads summarised in the same line")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run three device-to-device copies of 1 GiB (a kernel of known traffic, to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs the DP hot path on ONE GPU; --gpus must be 1 "
@@ -101,6 +110,20 @@ def main() -> int:
     def device_sync():
         if hip.hipDeviceSynchronize() != 0:
             raise RuntimeError("hipDeviceSynchronize failed")
+
+    if a.calibrate_copy:
+        n = 1 << 30
+        src, dst = ctypes.c_void_p(), ctypes.c_void_p()
+        assert hip.hipMalloc(ctypes.byref(src), ctypes.c_size_t(n)) == 0
+        assert hip.hipMalloc(ctypes.byref(dst), ctypes.c_size_t(n)) == 0
+        assert hip.hipMemset(src, 1, ctypes.c_size_t(n)) == 0
+        for _ in range(3):
+            assert hip.hipMemcpy(dst, src, ctypes.c_size_t(n), 3) == 0      # hipMemcpyDeviceToDevice
+        device_sync()
+        hip.hipFree(src)
+        hip.hipFree(dst)
+        print(json.dumps({"calibrate_copy_bytes": n, "copies": 3}))
+        return 0
 
     def measure(workload, steps, warmup):
         insts, probs = _problems(workload)
@@ -126,6 +149,8 @@ def main() -> int:
             "tflops": 3.0 * relax / launches / avg_launch_s / 1e12,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
+            "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
+            "kernel": "gdp_relax_fused_kernel" if tm.fused else "gdp_relax_kernel",
         }
 
     m = measure(a.workload, a.steps, a.warmup)
@@ -138,10 +163,11 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
-                   "mark_bytes": 1, "search_wall_ms_device": m["device_ms"], "device": _lib.device_info()},
+                   "mark_bytes": 1, "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
+                   "device": _lib.device_info()},
         "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
                      "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,
-                     "kernel": "gdp_relax_kernel", "launches_per_step": m["launches"],
+                     "kernel": m["kernel"], "launches_per_step": m["launches"],
                      "avg_launch_ms": m["avg_launch_ms"], "flops_per_relaxation": 3},
         "roofline_hbm": {"bound": "hbm", "achieved": m["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": m["gbs"] / PEAK_HBM_GBS, "traffic": traffic,
@@ -151,6 +177,7 @@ def main() -> int:
     for w in [x for x in a.also.split(",") if x and x != a.workload]:
         mm = measure(w, max(3, a.steps // 4), 1)
         also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
+                   "launch_scheme": mm["scheme"],
                    "roofline_frac_valu_fp64": mm["tflops"] / PEAK_FP64_VALU_TFLOPS,
                    "roofline_frac_hbm": mm["gbs"] / PEAK_HBM_GBS, "avg_launch_ms": mm["avg_launch_ms"]}
     if also:

@@ -530,6 +530,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
         t->relaxations = pl->relaxations;
         t->relax_bytes = pl->relax_bytes;
         t->relax_launches = (int32_t)launches;
+        t->fused = pl->fused ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));
         if (mode >= 2) {
             float sum = 0;

@@ -56,7 +56,7 @@ class gdp_result(ctypes.Structure):
 
 class gdp_timing(ctypes.Structure):
     _fields_ = [("total_ms", ctypes.c_float), ("relax_ms", ctypes.c_float), ("relax_launches", ctypes.c_int32),
-                ("reserved", ctypes.c_int32), ("relaxations", ctypes.c_double), ("relax_bytes", ctypes.c_double)]
+                ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("relax_bytes", ctypes.c_double)]
 
 
 _lib = None

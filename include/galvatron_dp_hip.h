@@ -84,7 +84,7 @@ typedef struct gdp_timing {
     float total_ms;        /* first kernel to last kernel (relaxation layers + epilogue)      */
     float relax_ms;        /* sum of the per-launch durations of the relaxation kernel         */
     int32_t relax_launches;
-    int32_t reserved;
+    int32_t fused;         /* 1: all layers in one launch, 0: one launch per layer             */
     double relaxations;    /* sum over instances of L*V*S*S                                    */
     double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write) */
 } gdp_timing;
