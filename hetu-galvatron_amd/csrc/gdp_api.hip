@@ -95,6 +95,8 @@ struct gdp_plan {
     std::vector<GdpDevOut> h_out;
     std::vector<int32_t> h_res;
     double relaxations = 0, relax_bytes = 0;
+    double executed = 0;     // relaxations actually carried out (tiles inside the bands)
+    bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
     bool ran = false;
     bool fused = true;            // one launch for all layers (work queue) instead of one per layer
     int64_t spin_limit = 1 << 22; // polls a waiting wave makes before the launch is abandoned
@@ -178,6 +180,52 @@ void destroy(gdp_plan *pl)
     delete pl;
 }
 
+// Per layer: how far down a reader reaches, and the band of tiles that has to be computed.
+//  lo: source rows u < reach = sum_{k<l} min{mem[k][s] : mem < V, intra finite} hold +inf for every
+//      strategy (by induction over the layers), so tiles entirely below `reach` need no arithmetic.
+//  hi: a cell written from source row u at layer l lies on a path to start row v0 only if
+//      u + sum_{k>=l} mem[k][s_k] = v0 for some choice, hence u <= max v0 - sum_{k>=l} min_s mem[k][s];
+//      rows above are never read by a row inside the band of the next layer, nor by the epilogue.
+// `skip` off (or exports requested, for hi) gives the full range.
+void fill_bands(const gdp_problem *q, const HostInst &h, int tile_rows, bool skip, int32_t *dep, double *executed)
+{
+    std::vector<int64_t> minfin((size_t)h.L), minany((size_t)h.L);
+    for (int l = 0; l < h.L; ++l) {
+        int maxm = 0;
+        int64_t mf = h.V, ma = h.V;
+        for (int s = 0; s < h.S; ++s) {
+            const int m = q->mem[(size_t)l * h.S + s];
+            if (m >= h.V) continue;
+            maxm = std::max(maxm, m);
+            ma = std::min<int64_t>(ma, m);
+            if (q->intra[(size_t)l * h.S + s] < INFINITY) mf = std::min<int64_t>(mf, m);
+        }
+        minfin[(size_t)l] = mf;
+        minany[(size_t)l] = ma;
+        dep[3 * l] = (maxm + tile_rows - 1) / tile_rows;
+    }
+    int64_t v0max = -1;
+    for (int k = 0; k < h.n_key; ++k) v0max = std::max<int64_t>(v0max, (int64_t)h.V - 1 - q->other_mem[k]);
+    const bool full = !skip || (h.flags & (GDP_EXPORT_F | GDP_EXPORT_MARK));
+    int64_t reach = 0;  // first row of the previous layer's output that can be finite
+    std::vector<int64_t> ub((size_t)h.L + 1);
+    ub[(size_t)h.L] = v0max;
+    for (int l = h.L - 1; l >= 0; --l) ub[(size_t)l] = ub[(size_t)l + 1] - minany[(size_t)l];
+    for (int l = 0; l < h.L; ++l) {
+        int64_t lo = skip ? std::min<int64_t>(reach, h.V) / tile_rows : 0;
+        int64_t hi = h.ntile - 1;
+        if (!full) hi = ub[(size_t)l] < 0 ? -1 : std::min<int64_t>(hi, ub[(size_t)l] / tile_rows);
+        if (lo > h.ntile) lo = h.ntile;
+        dep[3 * l + 1] = (int32_t)lo;
+        dep[3 * l + 2] = (int32_t)hi;  // -1: nothing to compute
+        if (hi >= lo) {
+            const int64_t rows = std::min<int64_t>(h.V, (hi + 1) * tile_rows) - lo * tile_rows;
+            *executed += (double)std::max<int64_t>(rows, 0) * (double)h.S * h.S;
+        }
+        reach = std::min<int64_t>(reach + minfin[(size_t)l], h.V);
+    }
+}
+
 int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
 {
     pl->n = n;
@@ -189,6 +237,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         fused_preset = true;
     }
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
+    if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_SPIN_LIMIT")) {
         const long long v = atoll(e);
@@ -270,6 +319,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         pl->groups.push_back(g);
         i = j;
     }
+    for (int i = 0; i < n; ++i)
+        if (p[i]->flags & GDP_COMPUTE_ALL) pl->skip = false;
     for (int i = 0; i < n && !fused_preset; ++i) {  // an explicit request of the caller
         if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
         else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
@@ -310,7 +361,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
         h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_UNROLL));
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
-        h.off_dep = take(sizeof(int32_t) * (size_t)h.L);
+        h.off_dep = take(sizeof(int32_t) * (size_t)h.L * 3);
     }
     const size_t small_bytes = off;
     // words that every run resets to zero: abort flag, ticket counters, completion counters
@@ -403,16 +454,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
             }
             for (int s = h.S; s < rows; ++s) row[s] = inf_row;  // padding sources and prefetch targets
         }
-        // dep[l]: a reader of layer l's output at tile t touches tiles [t - dep[l], t]
+        // dep[l] = {tiles a reader reaches down, first tile to compute, last tile to compute}
         int32_t *dep = reinterpret_cast<int32_t *>(stage.data() + h.off_dep);
-        for (int l = 0; l < h.L; ++l) {
-            int maxm = 0;
-            for (int s = 0; s < h.S; ++s) {
-                const int m = q->mem[(size_t)l * h.S + s];
-                if (m < h.V) maxm = std::max(maxm, m);
-            }
-            dep[l] = (maxm + tile_rows - 1) / tile_rows;
-        }
+        fill_bands(q, h, tile_rows, pl->skip, dep, &pl->executed);
         for (int k = 0; k < h.n_key; ++k) {
             GdpDevKey &key = dk[h.key_begin + k];
             key.other_mem = q->other_mem[k];
@@ -528,6 +572,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     if (t) {
         memset(t, 0, sizeof *t);
         t->relaxations = pl->relaxations;
+        t->executed = pl->executed;
         t->relax_bytes = pl->relax_bytes;
         t->relax_launches = (int32_t)launches;
         t->fused = pl->fused ? 1 : 0;

@@ -23,6 +23,13 @@
 //          padded with zeros up to SP = a multiple of the target tile).
 //   intra  L rows of SP doubles (zero padded).
 //   mem    L rows of S int32, as given.
+//   dep    L rows of 3 int32: {dep, lo, hi}.  dep = ceil(max mem[l] / tile rows): a reader of layer
+//          l's output at tile t touches tiles [t-dep, t].  lo/hi: the band of tiles of layer l that
+//          has to be computed.  Source rows below sum_{k<l} min_s mem[k][s] hold only +inf, so tiles
+//          entirely below are filled with +inf / argmin 0 without arithmetic (bit-identical to
+//          computing them).  Source rows above max start row - sum_{k>=l} min_s mem[k][s] cannot lie
+//          on any path that ends at a requested start row; they are skipped unless the caller asked
+//          for the full f / mark arrays.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -39,7 +46,8 @@ struct GdpDevInst {
     const int32_t *inter_index;
     const int64_t *roff;
     const int32_t *mem;
-    const int32_t *dep;  // [L] tiles below a tile that a reader of layer l's output needs
+    const int32_t *dep;  // [L][3]: tiles below a tile that a reader of layer l's output needs; first and
+                         // last tile of layer l that has to be computed (see tile_task)
     int64_t ld;          // elements per row of H
     int64_t ldm;         // entries per row of M
     int32_t L, V, S, SP;

@@ -151,6 +151,55 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
     }
 }
 
+// A tile whose source rows all lie below the first row that can hold a finite cost: every
+// candidate is +inf, so the cell is +inf and its argmin 0 (all-equal candidates go to index 0,
+// csrc/dp_core.cpp:12-16,70).  Same stores as relax_task, no arithmetic.
+template <int TS, int R, bool PUBLISH>
+__device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
+{
+    const int S = uload(&I->S);
+    const int P = uload(&I->P);
+    const int64_t ld = uload(&I->ld);
+    const int64_t ldm = uload(&I->ldm);
+    const int nbuf = uload(&I->nbuf);
+    double *dst = uload(&I->H) + (int64_t)((layer + 1) % nbuf) * uload(&I->hstride);
+    uint8_t *M = uload(&I->M);
+    const int s0 = tb * TS;
+    const int64_t u0 = (int64_t)tile * (64 * R);
+#pragma unroll
+    for (int j = 0; j < TS; ++j) {
+        const int s = s0 + j;
+        if (s < S) {
+            double *drow = dst + (int64_t)s * ld + P + u0;
+            uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (PUBLISH)
+                    __hip_atomic_store(drow + (lane + 64u * r), (double)INFINITY, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    drow[lane + 64u * r] = INFINITY;
+                mrow[lane + 64u * r] = 0;
+            }
+        }
+    }
+}
+
+// Rows of a layer that have to be computed (band[3*l+1] .. band[3*l+2], in tiles): below the band
+// every source cell is +inf (fill_task); above it no cell can lie on a path that ends at one of
+// the requested start rows, so nothing is read from there later and nothing is written.
+template <int TS, int R, bool PUBLISH>
+__device__ __forceinline__ void tile_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
+{
+    const int32_t *band = uload(&I->dep) + 3 * layer;
+    const unsigned lo = (unsigned)uload(band + 1), hi = (unsigned)uload(band + 2);
+    if (tile > hi) return;
+    if (tile < lo)
+        fill_task<TS, R, PUBLISH>(I, layer, tile, tb, lane);
+    else
+        relax_task<TS, R, PUBLISH>(I, layer, tile, tb, lane);
+}
+
 // ---- one launch per layer ------------------------------------------------------------------------
 // __launch_bounds__(256, 4): register allocation is held to 4 resident blocks per CU (4 waves per
 // SIMD, at most 128 VGPRs).
@@ -162,11 +211,26 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_kernel(
     if (layer >= uload(&I->L)) return;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned lane = threadIdx.x & 63u;
-    const unsigned task = xcd_swizzle(blockIdx.x, nblk_x) * GDP_WAVES_PER_BLOCK + wave;
-    const unsigned tile = task / ntb;
-    const unsigned tb = task - tile * ntb;
-    if (tile >= (unsigned)uload(&I->ntile)) return;
-    relax_task<TS, R, false>(I, layer, tile, tb, lane);
+    // Only the tiles lo..hi of this layer carry arithmetic.  The first blocks of the grid share them
+    // out, every XCD getting one contiguous range of them (equal work per XCD, neighbouring budget
+    // rows in one L2); the blocks after those fill the tiles below lo; tiles above hi are left alone.
+    const int32_t *band = uload(&I->dep) + 3 * layer;
+    const int lo = uload(band + 1), hi = uload(band + 2);
+    const unsigned live_tasks = hi >= lo ? (unsigned)(hi - lo + 1) * ntb : 0u;
+    const unsigned live_blocks = ((live_tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK + 7u) & ~7u;
+    (void)nblk_x;
+    if (blockIdx.x < live_blocks) {
+        const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
+        if (task >= live_tasks) return;
+        const unsigned t = task / ntb;
+        relax_task<TS, R, false>(I, layer, (unsigned)lo + t, task - t * ntb, lane);
+    } else {
+        const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
+        const unsigned t = task / ntb;
+        const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
+        if ((int)t > top) return;
+        fill_task<TS, R, false>(I, layer, t, task - t * ntb, lane);
+    }
 }
 
 // ---- all layers in one launch --------------------------------------------------------------------
@@ -264,7 +328,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_k
                 int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / (unsigned)ntb);
                 if (t_hi >= ntile) t_hi = ntile - 1;
                 if (t_lo < ntile) {
-                    const int d = uload(uload(&I->dep) + layer - 1);
+                    const int d = uload(uload(&I->dep) + 3 * (layer - 1));
                     const int lo = t_lo - d < 0 ? 0 : t_lo - d;
                     const int32_t *cnt_prev =
                         cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile;
@@ -291,7 +355,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_k
         const unsigned tb = q - tile * (unsigned)ntb;
         if (tile >= (unsigned)uload(&I->ntile)) continue;  // wave-uniform; the barriers are per ticket
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the tile's loads after the wait
-        relax_task<TS, R, true>(I, layer, tile, tb, lane);
+        tile_task<TS, R, true>(I, layer, tile, tb, lane);  // tiles outside the band still count as done
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every write-through store acknowledged
         if (lane == 0)
@@ -472,7 +536,7 @@ static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_nt
     const unsigned ntb = (unsigned)(SP / TS);
     const unsigned tasks = (unsigned)max_ntile_rows * ntb;
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
-    nblk = (nblk + 7u) & ~7u;
+    nblk = ((nblk + 7u) & ~7u) + 8u;  // live blocks are rounded up to 8, the fill blocks come after them
     dim3 grid(nblk, (unsigned)n_inst, 1), block(64 * GDP_WAVES_PER_BLOCK, 1, 1);
     hipLaunchKernelGGL((gdp_relax_kernel<TS, R>), grid, block, 0, stream, insts, layer, ntb, nblk);
     return hipGetLastError();

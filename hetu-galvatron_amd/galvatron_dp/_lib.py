@@ -25,6 +25,7 @@ GDP_EXPORT_F = 1
 GDP_EXPORT_MARK = 2
 GDP_LAUNCH_FUSED = 4
 GDP_LAUNCH_PER_LAYER = 8
+GDP_COMPUTE_ALL = 16
 GDP_MAX_S = 256
 GDP_OPT_FUSED = 1
 GDP_OPT_SPIN_LIMIT = 2
@@ -56,7 +57,8 @@ class gdp_result(ctypes.Structure):
 
 class gdp_timing(ctypes.Structure):
     _fields_ = [("total_ms", ctypes.c_float), ("relax_ms", ctypes.c_float), ("relax_launches", ctypes.c_int32),
-                ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("relax_bytes", ctypes.c_double)]
+                ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("executed", ctypes.c_double),
+                ("relax_bytes", ctypes.c_double)]
 
 
 _lib = None
@@ -119,7 +121,8 @@ class Problem:
     dtypes/layouts the C ABI wants, plus the output arrays it will fill."""
 
     def __init__(self, mem, intra, inter, V: int, other_mem: Sequence[int], other_time: Sequence[float], *,
-                 inter_index=None, export_f: bool = False, export_mark: bool = False, launch: str | None = None):
+                 inter_index=None, export_f: bool = False, export_mark: bool = False, launch: str | None = None,
+                 compute_all: bool = False):
         self.mem = np.ascontiguousarray(mem, dtype=np.int32)
         if self.mem.ndim != 2:
             raise ValueError("mem must be [L,S]")
@@ -148,7 +151,8 @@ class Problem:
             raise ValueError("launch must be None, 'fused' or 'per_layer'")
         self.flags = ((GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0) |
                       (GDP_LAUNCH_FUSED if launch == "fused" else 0) |
-                      (GDP_LAUNCH_PER_LAYER if launch == "per_layer" else 0))
+                      (GDP_LAUNCH_PER_LAYER if launch == "per_layer" else 0) |
+                      (GDP_COMPUTE_ALL if compute_all else 0))
         if self.V < 1 or self.L < 1 or self.S < 1:
             raise ValueError("L, V and S must be >= 1")
         # outputs

@@ -47,6 +47,7 @@ extern "C" {
 #define GDP_EXPORT_MARK 2u /* write result.mark_out (argmin table, reference layout [L][V][S]) */
 #define GDP_LAUNCH_FUSED 4u     /* lay the plan out for, and use, ONE launch over all layers          */
 #define GDP_LAUNCH_PER_LAYER 8u /* one launch per layer (two cost buffers); default: chosen by size    */
+#define GDP_COMPUTE_ALL 16u     /* carry out every one of the L*V*S*S relaxations (see gdp_timing.executed) */
 
 /* One DP instance == one reference call.  Field <- reference argument (csrc/dp_core.cpp:24-35):
  *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),
@@ -86,6 +87,8 @@ typedef struct gdp_timing {
     int32_t relax_launches;
     int32_t fused;         /* 1: all layers in one launch, 0: one launch per layer             */
     double relaxations;    /* sum over instances of L*V*S*S                                    */
+    double executed;       /* relaxations actually carried out: cells whose sources are all +inf, and cells
+                              that no requested start row can reach back to, are not computed           */
     double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write) */
 } gdp_timing;
 

@@ -64,6 +64,29 @@ def test_both_launch_schemes_give_identical_arrays(golden, name, fused):
             assert H.sha(prob.mark_out) == rec["mark_sha256"]
 
 
+@pytest.mark.parametrize("launch", ["fused", "per_layer"])
+@pytest.mark.parametrize("name", ["cfg2_small", "cfg4_small", "galvatron_like", "infeasible_6", "cfg3_smallV_5"])
+def test_skipping_rows_changes_nothing(golden, name, launch):
+    """Rows whose sources are all +inf are filled, rows no start row can reach back to are left out:
+    same results as computing every cell, and fewer relaxations carried out."""
+    rec = golden[name]
+    inst = H.build_case(rec)
+    done = {}
+    for compute_all in (True, False):
+        prob = _problem(inst, launch=launch, compute_all=compute_all)
+        with _lib.Plan([prob]) as plan:
+            plan.set_option(_lib.GDP_OPT_POISON, 1)
+            t = plan.run(1)
+            plan.fetch()
+        _check_against_golden(prob, rec, f"{name} compute_all={compute_all}")
+        done[compute_all] = t.executed / t.relaxations
+    assert abs(done[True] - 1.0) < 1e-12 and done[False] <= 1.0
+    # with the full arrays requested only the +inf rows may be skipped, and the arrays stay identical
+    prob = _problem(inst, launch=launch, export_f=True, export_mark=True)
+    _lib.solve_batch([prob])
+    assert H.sha(prob.f_out) == rec["f_sha256"] and H.sha(prob.mark_out) == rec["mark_sha256"]
+
+
 def test_abandoned_fused_launch_falls_back_or_reports(golden):
     """A spin limit of 1 makes waiting wavefronts give up at once (forced from the host; every
     kernel still runs to completion).  With the fallback the plan switches to per-layer launches
