@@ -1,0 +1,91 @@
+"""Differential test on the GPU: seeded random instances through the plugin signature against
+the C oracle, on shapes chosen to hit the kernel's corners: S around the register-tile widths
+(8, 11) and the wavefront width (63..65, 127..129, 255, 256), V not a multiple of any tile height,
+memory costs near 1, near V and above V, +inf costs, exact ties, shared and per-layer inter
+matrices, start rows below 0.  Full f and mark arrays are compared as well as the results."""
+import numpy as np
+import pytest
+
+import helpers as H
+from galvatron_dp import _lib, workloads as W
+from oracle import dp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 1, 1), (1, 1, 7), (2, 1, 64), (3, 2, 65), (4, 7, 191), (3, 8, 192), (5, 9, 193), (2, 10, 255),
+          (6, 11, 256), (3, 12, 257), (4, 16, 383), (2, 21, 385), (7, 22, 512), (3, 23, 700), (2, 33, 129),
+          (3, 44, 1000), (2, 45, 130), (2, 63, 300), (3, 64, 333), (2, 65, 200), (2, 88, 410), (1, 127, 150),
+          (2, 128, 140), (2, 129, 131), (1, 255, 90), (2, 256, 70), (9, 5, 2048), (12, 3, 4099), (20, 4, 1500)]
+
+
+def _compare(inst, tag, launch=None):
+    keys = sorted(inst.other_mem)
+    prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                        [inst.other_time[k] for k in keys], inter_index=inst.inter_index, export_f=True,
+                        export_mark=True, launch=launch)
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)
+        plan.run()
+        plan.fetch()
+    wt, wr, wm, wf, wmark = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time,
+                                    keep=True)
+    got = ({k: prob.total[i] for i, k in enumerate(keys)},
+           {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+           {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+    H.assert_same_results(got, (wt, wr, wm), tag)
+    assert prob.f_out.tobytes() == wf.tobytes(), f"{tag}: f differs"
+    assert np.array_equal(prob.mark_out, wmark), f"{tag}: mark differs"
+
+
+@pytest.mark.parametrize("n,shape", list(enumerate(SHAPES)))
+def test_random_instances_against_oracle(n, shape):
+    L, S, V = shape
+    for variant in range(4):
+        rng = np.random.Generator(np.random.PCG64([77, n, variant]))
+        ties = variant in (1, 3)
+        hi = [max(1, V // (L + 1)), max(1, V // 2), V + 3, 3][variant]
+        inst = W.random_instance(rng, L, S, V, integer_costs=ties, mem_hi=hi, per_layer_inter=bool(variant % 2),
+                                 inf_frac=0.2 if variant >= 2 else 0.0, over_frac=0.1 if variant == 3 else 0.0,
+                                 n_keys=min(4, 1 + variant))
+        _compare(inst, f"shape {shape} variant {variant}", launch=("fused", "per_layer", None, None)[variant])
+
+
+def test_no_keys_and_single_layer():
+    rng = np.random.Generator(np.random.PCG64(5))
+    inst = W.random_instance(rng, 1, 6, 50, mem_hi=20)
+    prob = _lib.Problem(inst.mem, inst.intra, inst.inter, 50, [], [], export_f=True)
+    _lib.solve_batch([prob])
+    wf = O.solve(inst.mem, inst.intra, inst.inter, 50, {}, {}, keep=True)[3]
+    assert prob.f_out.tobytes() == wf.tobytes()
+
+
+def test_start_row_outside_the_table():
+    rng = np.random.Generator(np.random.PCG64(6))
+    inst = W.random_instance(rng, 3, 4, 40, mem_hi=5)
+    inst.other_mem = {1: 0, 2: 39, 3: 40, 4: 10 ** 9}
+    inst.other_time = {k: 1.0 for k in inst.other_mem}
+    _compare(inst, "start rows 39, -1, far below 0")
+
+
+def test_many_threads_share_the_library():
+    """ctypes releases the GIL; concurrent calls from several threads must not disturb each other."""
+    import threading
+    rng = np.random.Generator(np.random.PCG64(8))
+    insts = [W.random_instance(rng, 4 + i % 3, 10 + i, 600 + 37 * i, mem_hi=60) for i in range(12)]
+    want = [O.solve(i.mem, i.intra, i.inter, i.V, i.other_mem, i.other_time) for i in insts]
+    errors = []
+
+    def work(k):
+        try:
+            for _ in range(3):
+                got = H.hip_solve(insts[k])
+                H.assert_same_results(got, want[k], f"thread {k}")
+        except Exception as e:  # noqa: BLE001
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(len(insts))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
