@@ -51,10 +51,11 @@ struct HostInst {
 };
 
 struct Group {  // instances with the same S, sorted by L descending
-    int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt, grid_blocks;
+    int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt;
     int64_t max_ld;
     std::vector<int> active;  // active[l] = number of instances with L > l
-    size_t off_sched, off_active, off_next, off_cnt;  // byte offsets in the device allocation
+    std::vector<std::pair<int, int>> segments;  // fused launches: (first layer, layers), same active set
+    size_t off_sched, off_active, off_cnt;  // byte offsets in the device allocation
 };
 
 // Target-tile width: the one that pads S the least (ties: the first).
@@ -326,13 +327,13 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
     }
     if (!fused_preset) {
-        // One launch for all layers pays off when a layer holds several times more block tasks than
-        // the device holds blocks: then the tasks a block waits for were finished long before, and
-        // its loads, stores and waits hide under the arithmetic of its neighbours.  A layer that
-        // barely fills the device is better off with a launch of its own.
+        // One launch for all layers pays off when a layer holds at least twice as many block tasks as
+        // the device holds blocks: then what a block waits for was finished a while ago, and its
+        // loads, stores and waits hide under the arithmetic of its neighbours.  Below that the
+        // latency of signalling through memory shows, and a launch per layer is quicker.
         int64_t first_layer = 0;
         for (const Group &g : pl->groups) first_layer += (int64_t)g.active[0] * g.nbt;
-        pl->fused = first_layer >= 4 * (int64_t)pl->num_cu * 4;
+        pl->fused = first_layer >= 2 * (int64_t)pl->num_cu * 4;
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -368,7 +369,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     pl->off_zero = off;
     pl->off_abort = take(sizeof(int32_t));
     for (auto &g : pl->groups) {
-        g.off_next = take(sizeof(int32_t) * (size_t)g.max_L);
         g.off_cnt = take(sizeof(int32_t) * (size_t)g.count * g.max_L * g.max_ntile);
     }
     pl->zero_words = (off - pl->off_zero) / sizeof(int32_t);
@@ -469,7 +469,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     }
     for (auto &g : pl->groups) {
         GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
-        sc->next = reinterpret_cast<int32_t *>(pl->dbase + g.off_next);
         sc->cnt = reinterpret_cast<int32_t *>(pl->dbase + g.off_cnt);
         sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
@@ -481,14 +480,24 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
             act[l] = g.active[(size_t)l];
             tasks += (int64_t)g.active[(size_t)l] * g.nbt;
         }
-        int per_cu = 1;
-        GDP_HIP(gdp_fused_blocks_per_cu(g.variant, &per_cu));
-        const int64_t first_layer = (int64_t)g.active[0] * g.nbt;
-        int want = 4;  // resident blocks per CU (16 waves, 4 per SIMD)
-        if (const char *e = getenv("GALVATRON_DP_BLOCKS_PER_CU")) want = std::max(1, atoi(e));
-        int64_t grid = std::min<int64_t>(first_layer, (int64_t)std::max(std::min(per_cu, want), 1) * pl->num_cu);
-        g.grid_blocks = (int)std::max<int64_t>(1, grid);
         (void)tasks;
+        // One fused launch per run of layers with the same number of active instances (grid.y <= 65535);
+        // a batch with very many different depths merges the shortest runs into their predecessors.
+        g.segments.clear();
+        for (int l = 0; l < g.max_L; ++l) {
+            if (!g.segments.empty() && g.active[(size_t)l] == g.active[(size_t)g.segments.back().first] &&
+                g.segments.back().second < 65535)
+                g.segments.back().second++;
+            else
+                g.segments.push_back({l, 1});
+        }
+        while (g.segments.size() > 32) {
+            size_t best = 1;
+            for (size_t i = 1; i < g.segments.size(); ++i)
+                if (g.segments[i].second < g.segments[best].second) best = i;
+            g.segments[best - 1].second += g.segments[best].second;
+            g.segments.erase(g.segments.begin() + (long)best);
+        }
     }
     GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));
     GDP_HIP(hipEventCreate(&pl->ev_begin));
@@ -515,7 +524,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
     int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
     size_t launches = 0;
-    for (const Group &g : pl->groups) launches += pl->fused ? 1 : (size_t)g.max_L;
+    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : (size_t)g.max_L;
     if (mode >= 2)
         while (pl->ev_relax.size() < 2 * launches) {
             hipEvent_t e;
@@ -533,14 +542,16 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     if (pl->fused) {
         GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
                                 pl->stream));
-        for (const Group &g : pl->groups) {
-            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-            GDP_HIP(gdp_launch_relax_fused(g.variant, d_insts + g.first,
-                                           reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), g.grid_blocks,
-                                           pl->stream));
-            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
-            ++li;
-        }
+        for (const Group &g : pl->groups)
+            for (const auto &seg : g.segments) {  // (first layer, number of layers)
+                const int grid_x = (int)align_up((size_t)std::max<int64_t>(1, (int64_t)g.active[(size_t)seg.first] * g.nbt), 8);
+                if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
+                GDP_HIP(gdp_launch_relax_fused(g.variant, d_insts + g.first,
+                                               reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,
+                                               seg.first, seg.second, pl->stream));
+                if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
+                ++li;
+            }
     } else {
         for (int l = 0; l < pl->max_L; ++l)
             for (const Group &g : pl->groups) {

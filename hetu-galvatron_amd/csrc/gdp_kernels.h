@@ -59,7 +59,6 @@ struct GdpDevInst {
 
 // Bookkeeping of one fused (all layers) launch over a group of instances.
 struct GdpSched {
-    int32_t *next;            // [max_L] ticket counter per layer                  (zeroed per run)
     int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
@@ -91,12 +90,10 @@ static const GdpVariant GDP_VARIANTS[] = {{8, 4}, {8, 2}, {8, 1}, {11, 3}, {11, 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
 hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
                             hipStream_t stream);
-// All layers of a group in one launch: blocks draw (layer, instance, tile) tasks from ticket
-// counters and wait on per-tile completion counters instead of on a kernel boundary.
+// Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
+// layers): a block waits on per-tile completion counters instead of on a kernel boundary.
 hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
-                                  hipStream_t stream);
-// Resident blocks per CU of the fused kernel (for sizing its grid).
-hipError_t gdp_fused_blocks_per_cu(int variant, int *blocks);
+                                  int layer0, int layers, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
 // in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).

@@ -267,18 +267,21 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
     return true;
 }
 
-// Blocks draw block tasks (four consecutive (tile, target block) wave tasks of one instance and
-// layer) from ticket counters, layer by layer: all tickets of layer l are handed out before any of
-// layer l+1.  Whatever a task waits for therefore was handed out earlier and is running or
-// finished, the oldest unfinished task never waits, and the launch cannot deadlock whatever the
-// residency of its blocks.  Drawing tickets (rather than owning a fixed share) also keeps the four
-// waves of a SIMD out of step with each other, so that one wave's loads, stores and waits are
-// covered by the arithmetic of the others.
+// One launch for a run of layers (all of them, unless instances of different depth share the
+// batch: then one launch per run of layers with the same set of active instances, so that no
+// launch carries empty workgroups): grid.y = layer - layer0, grid.x = block task (four consecutive
+// (tile, target block) wave tasks of one instance).  Workgroups are dispatched in order of their linear id, x
+// fastest, so every block of layer l is dispatched before any block of layer l+1; a block only
+// ever waits for blocks of the layer before its own, which therefore run or have finished, and the
+// oldest unfinished block never waits: the launch cannot deadlock.  (Each XCD takes every eighth
+// workgroup and dispatches its share in order, which is all the argument needs.)  Older workgroups
+// also win the issue arbitration of their SIMD, so the work that others wait for runs first.
 //
 // Instead of a kernel boundary between layers, a task waits only for the tiles it reads: layer l,
 // tile t reads rows of layer l-1's output in tiles [t-dep[l-1], t].  Every layer has its own cost
 // buffer inside a fused launch, so nothing is overwritten and read-after-write is the only
-// dependence.
+// dependence.  Waits are bounded; if one runs out the launch drains and the host repeats the solve
+// with one launch per layer.
 //
 // Visibility across the 8 XCDs, whose L2s are not coherent with each other:
 //  - a cost cell is written once per launch with a write-through (agent scope) store, the writer
@@ -288,80 +291,60 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //    before its counter is full, and the caches are invalidated when the launch begins.
 template <int TS, int R>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_kernel(
-    const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q)
+    const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q, int layer0)
 {
-    __shared__ int sh_ticket[2];
+    __shared__ int sh_ok;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned lane = threadIdx.x & 63u;
+    const int layer = layer0 + (int)blockIdx.y;
     const int max_L = uload(&Q->max_L);
     const int max_ntile = uload(&Q->max_ntile);
     const int ntb = uload(&Q->ntb);
     const int nbt = uload(&Q->nbt);
-    int32_t *next = uload(&Q->next);
+    const int nat = uload(uload(&Q->n_active) + layer);
+    // The grid is as wide as the fullest layer.  Inside a layer the first `total8` workgroups share
+    // out its block tasks, every XCD getting one contiguous range of them; the rest have nothing to do.
+    const unsigned total = (unsigned)(nat * nbt);
+    const unsigned total8 = (total + 7u) & ~7u;
+    if (blockIdx.x >= total8) return;
+    const unsigned x = xcd_swizzle(blockIdx.x, total8);
+    if (x >= total) return;
     int32_t *cnt_all = uload(&Q->cnt);
     int32_t *abort_flag = uload(&Q->abort_flag);
-    const int32_t *n_active = uload(&Q->n_active);
-    const int64_t limit = uload(&Q->spin_limit);
-    int layer = 0;
-    for (;;) {
-        // ---- wave 0 draws the next ticket and waits for what the block's four wave tasks read -----
+    const int bt = (int)(x / (unsigned)nat);  // block task within the instance: tiles ascend with x
+    const int ii = (int)x - bt * nat;         // instance (a prefix of the table is active)
+    const GdpDevInst *I = insts + ii;
+    const int ntile = uload(&I->ntile);
+    const unsigned q0 = (unsigned)bt * GDP_WAVES_PER_BLOCK;
+    if (layer >= 1) {
+        // the block's first wave waits for everything its four wave tasks read
         if (wave == 0) {
-            int ticket = -1;
-            while (layer < max_L) {
-                const int total = uload(n_active + layer) * nbt;
-                int k = 0;
-                if (lane == 0)
-                    k = __hip_atomic_fetch_add(next + layer, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ticket = __builtin_amdgcn_readfirstlane(k);
-                if (ticket < total) break;
-                ticket = -1;
-                ++layer;
+            const int t_lo = (int)(q0 / (unsigned)ntb);
+            int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / (unsigned)ntb);
+            if (t_hi >= ntile) t_hi = ntile - 1;
+            bool ok = true;
+            if (t_lo < ntile) {
+                const int d = uload(uload(&I->dep) + 3 * (layer - 1));
+                const int lo = t_lo - d < 0 ? 0 : t_lo - d;
+                ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, lo, t_hi, ntb, lane,
+                                abort_flag, uload(&Q->spin_limit));
             }
-            if (ticket >= 0 && layer >= 1) {
-                const int nat = uload(n_active + layer);
-                const int bt = ticket / nat;
-                const int ii = ticket - bt * nat;
-                const GdpDevInst *I = insts + ii;
-                const int ntile = uload(&I->ntile);
-                const unsigned q0 = (unsigned)bt * GDP_WAVES_PER_BLOCK;
-                const int t_lo = (int)(q0 / (unsigned)ntb);
-                int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / (unsigned)ntb);
-                if (t_hi >= ntile) t_hi = ntile - 1;
-                if (t_lo < ntile) {
-                    const int d = uload(uload(&I->dep) + 3 * (layer - 1));
-                    const int lo = t_lo - d < 0 ? 0 : t_lo - d;
-                    const int32_t *cnt_prev =
-                        cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile;
-                    if (!wait_tiles(cnt_prev, lo, t_hi, ntb, lane, abort_flag, limit)) ticket = -1;
-                }
-            }
-            if (ticket >= 0 && __builtin_amdgcn_readfirstlane(ld_agent(abort_flag)) != 0) ticket = -1;
-            if (lane == 0) {
-                sh_ticket[0] = ticket;
-                sh_ticket[1] = layer;
-            }
+            if (lane == 0) sh_ok = ok ? 1 : 0;
         }
         __syncthreads();
-        const int ticket = __builtin_amdgcn_readfirstlane(sh_ticket[0]);
-        layer = __builtin_amdgcn_readfirstlane(sh_ticket[1]);
-        __syncthreads();  // sh_ticket is rewritten only after every wave has read it
-        if (ticket < 0) return;  // out of work, or the launch is being abandoned (block-uniform)
-        const int nat = uload(n_active + layer);
-        const int bt = ticket / nat;       // block task within the instance: tiles ascend with tickets
-        const int ii = ticket - bt * nat;  // instance (a prefix of the table is active)
-        const GdpDevInst *I = insts + ii;
-        const unsigned q = (unsigned)bt * GDP_WAVES_PER_BLOCK + wave;
-        const unsigned tile = q / (unsigned)ntb;
-        const unsigned tb = q - tile * (unsigned)ntb;
-        if (tile >= (unsigned)uload(&I->ntile)) continue;  // wave-uniform; the barriers are per ticket
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the tile's loads after the wait
-        tile_task<TS, R, true>(I, layer, tile, tb, lane);  // tiles outside the band still count as done
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every write-through store acknowledged
-        if (lane == 0)
-            __hip_atomic_fetch_add(cnt_all + ((int64_t)ii * max_L + layer) * max_ntile + tile, 1, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+        if (__builtin_amdgcn_readfirstlane(sh_ok) == 0) return;  // the launch is being abandoned
     }
+    const unsigned q = q0 + wave;
+    const unsigned tile = q / (unsigned)ntb;
+    const unsigned tb = q - tile * (unsigned)ntb;
+    if (tile >= (unsigned)ntile) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the tile's loads after the wait
+    tile_task<TS, R, true>(I, layer, tile, tb, lane);        // tiles outside the band still count as done
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // every write-through store acknowledged
+    if (lane == 0)
+        __hip_atomic_fetch_add(cnt_all + ((int64_t)ii * max_L + layer) * max_ntile + tile, 1, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __global__ __launch_bounds__(256) void gdp_zero_kernel(int32_t *p, int64_t n)
@@ -558,30 +541,19 @@ hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, in
 }
 
 hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
-                                  hipStream_t stream)
+                                  int layer0, int layers, hipStream_t stream)
 {
-    dim3 grid((unsigned)grid_blocks), block(64 * GDP_WAVES_PER_BLOCK);
-#define X(id, ts, r) \
-    case id: hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r>), grid, block, 0, stream, insts, sched); break;
+    dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
+#define X(id, ts, r)                                                                                       \
+    case id:                                                                                               \
+        hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r>), grid, block, 0, stream, insts, sched, layer0); \
+        break;
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
     }
 #undef X
     return hipGetLastError();
-}
-
-hipError_t gdp_fused_blocks_per_cu(int variant, int *blocks)
-{
-#define X(id, ts, r)                                                                                 \
-    case id:                                                                                         \
-        return hipOccupancyMaxActiveBlocksPerMultiprocessor(blocks, gdp_relax_fused_kernel<ts, r>, \
-                                                            64 * GDP_WAVES_PER_BLOCK, 0);
-    switch (variant) {
-        GDP_FOR_EACH_VARIANT(X)
-        default: return hipErrorInvalidValue;
-    }
-#undef X
 }
 
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)
