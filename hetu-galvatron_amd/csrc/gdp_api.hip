@@ -99,7 +99,9 @@ struct gdp_plan {
     double executed = 0;     // relaxations actually carried out (tiles inside the bands)
     bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
     bool ran = false;
-    bool fused = true;            // one launch for all layers (work queue) instead of one per layer
+    bool fused = true;            // one launch for all layers instead of one per layer
+    bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
+                                  // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
     int64_t spin_limit = 1 << 22; // polls a waiting wave makes before the launch is abandoned
     size_t off_zero = 0, zero_words = 0, off_abort = 0;
     int num_cu = 0;
@@ -237,6 +239,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         pl->fused = atoi(e) != 0;
         fused_preset = true;
     }
+    bool marks_preset = false;
+    if (const char *e = getenv("GALVATRON_DP_KEEP_MARKS")) {
+        pl->keep_marks = atoi(e) != 0;
+        marks_preset = true;
+    }
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
@@ -320,8 +327,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         pl->groups.push_back(g);
         i = j;
     }
-    for (int i = 0; i < n; ++i)
+    for (int i = 0; i < n; ++i) {
         if (p[i]->flags & GDP_COMPUTE_ALL) pl->skip = false;
+        if ((p[i]->flags & GDP_KEEP_MARKS) && !marks_preset) pl->keep_marks = true;
+        if (p[i]->flags & GDP_EXPORT_MARK) pl->keep_marks = true;  // the table itself is asked for
+    }
     for (int i = 0; i < n && !fused_preset; ++i) {  // an explicit request of the caller
         if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
         else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
@@ -357,10 +367,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         g.off_active = take(sizeof(int32_t) * (size_t)g.max_L);
     }
     for (auto &h : inst) {
-        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_UNROLL) * h.SP);
+        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_PAD) * h.SP);
         h.off_intra = take(sizeof(double) * (size_t)h.L * h.SP);
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
-        h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_UNROLL));
+        h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_PAD));
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
         h.off_dep = take(sizeof(int32_t) * (size_t)h.L * 3);
     }
@@ -375,25 +385,27 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     pl->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(nk, 1));
     pl->off_res = take(sizeof(int32_t) * std::max<size_t>(nres, 1));
     const size_t fixed_bytes = off;
-    // One cost buffer per layer lets all layers share a launch; if that does not fit in device
-    // memory, fall back to two buffers and one launch per layer.
+    // One cost buffer per layer lets all layers share a launch and lets the backtrack recompute the
+    // argmin of the cells it visits, so that the relaxation does not have to track it.  If that does
+    // not fit in device memory: two cost buffers, the argmin table, one launch per layer.
     for (int attempt = 0; attempt < 2; ++attempt) {
         off = fixed_bytes;
-        pl->can_fuse = pl->fused;
+        pl->can_fuse = pl->fused || !pl->keep_marks;
         pl->rezero = false;
         for (auto &h : inst) {
-            h.nbuf = pl->fused ? h.L + 1 : 2;
+            h.nbuf = pl->can_fuse ? h.L + 1 : 2;
             if (h.nbuf < h.L + 1) pl->rezero = true;
             h.off_H = take(sizeof(double) * (size_t)h.nbuf * (size_t)(h.S + 1) * (size_t)h.ld);
-            h.off_M = take((size_t)h.L * h.S * (size_t)h.ldm);
+            h.off_M = pl->keep_marks ? take((size_t)h.L * h.S * (size_t)h.ldm) : 0;
         }
         pl->dbytes = off;
         hipError_t e = hipMalloc((void **)&pl->dbase, pl->dbytes);
         if (e == hipSuccess) break;
         pl->dbase = nullptr;
         (void)hipGetLastError();
-        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->fused) {
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse) {
             pl->fused = false;
+            pl->keep_marks = true;
             continue;
         }
         char buf[128];
@@ -416,7 +428,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         d.H = reinterpret_cast<double *>(pl->dbase + h.off_H);
         d.hstride = (int64_t)(h.S + 1) * h.ld;
         d.nbuf = h.nbuf;
-        d.M = reinterpret_cast<uint8_t *>(pl->dbase + h.off_M);
+        d.M = pl->keep_marks ? reinterpret_cast<uint8_t *>(pl->dbase + h.off_M) : nullptr;
         d.inter = reinterpret_cast<const double *>(pl->dbase + h.off_inter);
         d.intra = reinterpret_cast<const double *>(pl->dbase + h.off_intra);
         d.inter_index = reinterpret_cast<const int32_t *>(pl->dbase + h.off_index);
@@ -425,7 +437,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         d.dep = reinterpret_cast<const int32_t *>(pl->dbase + h.off_dep);
         d.ld = h.ld; d.ldm = h.ldm;
         d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.SU = h.SU; d.P = h.P; d.ntile = h.ntile;
-        const int rows = h.SU + GDP_SRC_UNROLL;  // source rows per matrix / offsets per layer
+        const int rows = h.SU + GDP_SRC_PAD;  // source rows per matrix / offsets per layer
         const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
         // inter: [T][rows][SP], zero padded
         double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
@@ -465,22 +477,18 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
             key.res_off = h.res_begin + k * h.L;
         }
         pl->relaxations += (double)h.L * h.V * (double)h.S * h.S;
-        pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + 1);
+        pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + (pl->keep_marks ? 1 : 0));
     }
     for (auto &g : pl->groups) {
         GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
         sc->cnt = reinterpret_cast<int32_t *>(pl->dbase + g.off_cnt);
         sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
-        sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb; sc->nbt = g.nbt;
+        sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb;
+        sc->slots = (g.nbt + 7) / 8 + 1;
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
-        int64_t tasks = 0;
-        for (int l = 0; l < g.max_L; ++l) {
-            act[l] = g.active[(size_t)l];
-            tasks += (int64_t)g.active[(size_t)l] * g.nbt;
-        }
-        (void)tasks;
+        for (int l = 0; l < g.max_L; ++l) act[l] = g.active[(size_t)l];
         // One fused launch per run of layers with the same number of active instances (grid.y <= 65535);
         // a batch with very many different depths merges the shortest runs into their predecessors.
         g.segments.clear();
@@ -544,9 +552,10 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                                 pl->stream));
         for (const Group &g : pl->groups)
             for (const auto &seg : g.segments) {  // (first layer, number of layers)
-                const int grid_x = (int)align_up((size_t)std::max<int64_t>(1, (int64_t)g.active[(size_t)seg.first] * g.nbt), 8);
+                // per XCD and instance: an eighth of the block tasks inside the band and an eighth of the rest
+                const int grid_x = 8 * g.active[(size_t)seg.first] * ((g.nbt + 7) / 8 + 1);
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax_fused(g.variant, d_insts + g.first,
+                GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks, d_insts + g.first,
                                                reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,
                                                seg.first, seg.second, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
@@ -557,13 +566,13 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
             for (const Group &g : pl->groups) {
                 if (l >= g.max_L) continue;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax(g.variant, d_insts + g.first, g.active[(size_t)l], g.max_ntile, g.SP, l,
-                                         pl->stream));
+                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, d_insts + g.first, g.active[(size_t)l], g.max_ntile,
+                                         g.SP, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
     }
-    GDP_HIP(gdp_launch_epilogue(d_insts, d_keys, pl->n_key_total, d_out, d_res, pl->stream));
+    GDP_HIP(gdp_launch_epilogue(pl->keep_marks, d_insts, d_keys, pl->n_key_total, d_out, d_res, pl->stream));
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
     int32_t aborted = 0;
     if (pl->fused)

@@ -14,12 +14,14 @@
 //          (csrc/dp_core.cpp:60-64) without a branch.  Row S is +inf everywhere and stands in
 //          for strategies whose mem reaches V and for the padding source strategies.
 //   M      argmin table, L*S rows of `ldm` entries (one byte each), indexed by the SOURCE row u
-//          like H: mark[l][v][s] of the reference is M[l][s][v - mem[l][s]].
-//   roff   (L+1) rows of SU+GDP_SRC_UNROLL int64: element offset, from the base of a cost buffer,
+//          like H: mark[l][v][s] of the reference is M[l][s][v - mem[l][s]].  Only present when the
+//          plan keeps marks; otherwise nbuf is L+1 and the backtrack recomputes the argmin of the
+//          cells on its path from H.
+//   roff   (L+1) rows of SU+GDP_SRC_PAD int64: element offset, from the base of a cost buffer,
 //          at which "f of the previous layer, strategy s', row 0" is found (SU = S rounded up to
 //          the source unroll; the entries from S on point at the +inf row: padding sources and the
 //          targets of the last prefetches).
-//   inter  n_inter matrices, each SU+GDP_SRC_UNROLL rows (rows >= S zero) of SP doubles (columns
+//   inter  n_inter matrices, each SU+GDP_SRC_PAD rows (rows >= S zero) of SP doubles (columns
 //          padded with zeros up to SP = a multiple of the target tile).
 //   intra  L rows of SP doubles (zero padded).
 //   mem    L rows of S int32, as given.
@@ -36,6 +38,7 @@
 
 #define GDP_WAVES_PER_BLOCK 4
 #define GDP_SRC_UNROLL 2  // source strategies are consumed two at a time (padded with +inf sources)
+#define GDP_SRC_PAD 4     // dummy source rows after SU in roff / inter: targets of the last prefetches
 
 struct GdpDevInst {
     double *H;        // buffer b starts at H + b * hstride
@@ -62,7 +65,8 @@ struct GdpSched {
     int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
-    int32_t max_L, max_ntile, ntb, nbt;  // nbt = block tasks per instance and layer
+    int32_t max_L, max_ntile, ntb;
+    int32_t slots;            // workgroups per XCD, instance and layer: ceil(block tasks / 8) + 1
     int64_t spin_limit;       // polls before a waiting wave gives up
 };
 
@@ -88,12 +92,13 @@ static const GdpVariant GDP_VARIANTS[] = {{8, 4}, {8, 2}, {8, 1}, {11, 3}, {11, 
 #define GDP_NUM_VARIANTS 6
 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
-hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
-                            hipStream_t stream);
+// marks: track and store the argmin table (otherwise costs only).
+hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevInst *insts, int n_inst, int max_ntile, int SP,
+                            int layer, hipStream_t stream);
 // Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
-hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
-                                  int layer0, int layers, hipStream_t stream);
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpDevInst *insts, const GdpSched *sched,
+                                  int grid_blocks, int layer0, int layers, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
 // in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).
@@ -104,8 +109,9 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
                            hipStream_t stream);
 // Fills n int32 with zero (queue counters; a kernel rather than a memset so that it can be captured).
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream);
-// argmin over the last layer's row + backtrack, one wavefront per key.
-hipError_t gdp_launch_epilogue(const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,
+// argmin over the last layer's row + backtrack, one wavefront per key (marks: through the stored
+// argmin table; otherwise recomputed from the cost buffers of all layers).
+hipError_t gdp_launch_epilogue(bool marks, const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,
                                int32_t *res, hipStream_t stream);
 // Debug exports in the reference's layouts.
 hipError_t gdp_launch_export_f(const GdpDevInst *inst, double *f_out, int V, int S, hipStream_t stream);

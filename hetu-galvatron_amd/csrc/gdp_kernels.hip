@@ -39,10 +39,34 @@ __device__ __forceinline__ unsigned xcd_swizzle(unsigned x, unsigned nblk)
     return (x & 7u) * (nblk >> 3) + (x >> 3);
 }
 
+// Nothing is moved across this point by the instruction scheduler.
+#define GDP_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Relaxations of target columns [J0, J1) of the register tile against one source strategy:
+// candidate = (f_prev + inter) + intra in that association (csrc/dp_core.cpp:68), strict '<' for the
+// argmin (csrc/dp_core.cpp:12-16).
+template <int TS, int R, bool ARG, int J0, int J1>
+__device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG ? R : 1][ARG ? TS : 1],
+                                           const double (&fp)[R], const double (&sc)[TS], const double (&add)[TS],
+                                           int sp)
+{
+#pragma unroll
+    for (int j = J0; j < J1; ++j)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const double c = (fp[r] + sc[j]) + add[j];
+            if constexpr (ARG) arg[r][j] = (c < best[r][j]) ? sp : arg[r][j];
+            best[r][j] = min_f64(best[r][j], c);
+        }
+}
+
 // One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of layer `layer`.
 // PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
 // waits for this task's completion counter finds them in memory.
-template <int TS, int R, bool PUBLISH>
+// ARG: also track and store the argmin (the reference's mark table, csrc/dp_core.cpp:70-72).  Without
+// it a relaxation is two additions and one minimum; the backtrack then recomputes the argmin of the
+// few cells on its path from the cost buffers, all of which are kept in that mode.
+template <int TS, int R, bool PUBLISH, bool ARG>
 __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb,
                                            unsigned lane)
 {
@@ -57,11 +81,11 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
     double *const hbase = uload(&I->H);
     const double *src = hbase + (int64_t)(layer % nbuf) * hstride;
     double *dst = hbase + (int64_t)((layer + 1) % nbuf) * hstride;
-    uint8_t *M = uload(&I->M);
-    const int64_t *ro = uload(&I->roff) + (int64_t)layer * (SU + GDP_SRC_UNROLL);
+    [[maybe_unused]] uint8_t *M = uload(&I->M);
+    const int64_t *ro = uload(&I->roff) + (int64_t)layer * (SU + GDP_SRC_PAD);
     const int s0 = tb * TS;
     const int mat = uload(uload(&I->inter_index) + layer);
-    const double *it = uload(&I->inter) + (int64_t)mat * (SU + GDP_SRC_UNROLL) * SP + s0;
+    const double *it = uload(&I->inter) + (int64_t)mat * (SU + GDP_SRC_PAD) * SP + s0;
     const double *ia = uload(&I->intra) + (int64_t)layer * SP + s0;
     const int64_t u0 = (int64_t)tile * (64 * R);
 
@@ -70,66 +94,82 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
     for (int j = 0; j < TS; ++j) add[j] = uload(ia + j);
 
     double best[R][TS];
-    int arg[R][TS];
+    int arg[ARG ? R : 1][ARG ? TS : 1];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int j = 0; j < TS; ++j) {
             best[r][j] = INFINITY;
-            arg[r][j] = 0;
+            if constexpr (ARG) arg[r][j] = 0;
         }
 
-    // Two register sets (A: even source strategies, B: odd) so that the loads for strategy sp+2 are
-    // in flight while strategy sp+1 is being consumed.  Entries SU, SU+1 of roff / inter are valid
-    // dummies, and source strategies in [S, SU) read the +inf row: +inf never wins a strict '<'.
+    // Software pipeline over the source strategies, two per trip (A: even, B: odd), with the order
+    // of issue pinned by scheduling fences, because every load has to be in flight for most of a
+    // half trip (TS*R cells) before its first use:
+    //   - the cost rows of strategy sp+2 are requested as soon as those of sp have been consumed,
+    //     i.e. a whole half trip before they are needed;
+    //   - the transition costs of the next strategy and the row offset of the one after it are
+    //     requested right after the first column of a half trip.  Scalar loads return out of order,
+    //     so waiting for one means waiting for all: after that first column nothing else is pending.
+    // Entries S.. of roff / inter are valid dummies (+inf row, zeros); +inf never wins.
     double fpA[R], fpB[R], scA[TS], scB[TS];
+    const double *itp = it;                    // row sp of the transition matrix
+    const int64_t *rop = ro;                   // roff[sp]
+    int64_t offA = uload(ro + 2), offB = uload(ro + 3);
     {
+        // same order of issue as inside the loop, so that the waits at the loop head count alike
+        // on both ways into it
         const double *pa = src + uload(ro) + u0;
         const double *pb = src + uload(ro + 1) + u0;
+        GDP_SCHED_FENCE();
 #pragma unroll
-        for (int r = 0; r < R; ++r) fpA[r] = pa[lane + 64u * r];
+        for (int r = 0; r < R; ++r) {
+            fpA[r] = pa[lane + 64u * r];
+            GDP_SCHED_FENCE();
+        }
 #pragma unroll
-        for (int r = 0; r < R; ++r) fpB[r] = pb[lane + 64u * r];
+        for (int r = 0; r < R; ++r) {
+            fpB[r] = pb[lane + 64u * r];
+            GDP_SCHED_FENCE();
+        }
 #pragma unroll
-        for (int j = 0; j < TS; ++j) scA[j] = uload(it + j);
-#pragma unroll
-        for (int j = 0; j < TS; ++j) scB[j] = uload(it + SP + j);
+        for (int j = 0; j < TS; ++j) scA[j] = uload(itp + j);
+        GDP_SCHED_FENCE();
     }
-
     const int S2 = (S + 1) & ~1;
     for (int sp = 0; sp < S2; sp += 2) {
+        relax_cols<TS, R, ARG, 0, 1>(best, arg, fpA, scA, add, sp);
+        GDP_SCHED_FENCE();
 #pragma unroll
-        for (int j = 0; j < TS; ++j)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const double c = (fpA[r] + scA[j]) + add[j];
-                const bool lt = c < best[r][j];
-                best[r][j] = min_f64(best[r][j], c);
-                arg[r][j] = lt ? sp : arg[r][j];
-            }
+        for (int j = 0; j < TS; ++j) scB[j] = uload(itp + SP + j);
+        const int64_t offA2 = uload(rop + 4);
+        GDP_SCHED_FENCE();
+        relax_cols<TS, R, ARG, 1, TS>(best, arg, fpA, scA, add, sp);
+        GDP_SCHED_FENCE();
         {
-            const double *pn = src + uload(ro + sp + 2) + u0;
+            const double *pn = src + offA + u0;
 #pragma unroll
             for (int r = 0; r < R; ++r) fpA[r] = pn[lane + 64u * r];
-#pragma unroll
-            for (int j = 0; j < TS; ++j) scA[j] = uload(it + (int64_t)(sp + 2) * SP + j);
         }
+        GDP_SCHED_FENCE();
+        relax_cols<TS, R, ARG, 0, 1>(best, arg, fpB, scB, add, sp + 1);
+        GDP_SCHED_FENCE();
+        itp += 2 * (int64_t)SP;
 #pragma unroll
-        for (int j = 0; j < TS; ++j)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const double c = (fpB[r] + scB[j]) + add[j];
-                const bool lt = c < best[r][j];
-                best[r][j] = min_f64(best[r][j], c);
-                arg[r][j] = lt ? (sp + 1) : arg[r][j];
-            }
+        for (int j = 0; j < TS; ++j) scA[j] = uload(itp + j);
+        const int64_t offB2 = uload(rop + 5);
+        GDP_SCHED_FENCE();
+        relax_cols<TS, R, ARG, 1, TS>(best, arg, fpB, scB, add, sp + 1);
+        GDP_SCHED_FENCE();
         {
-            const double *pn = src + uload(ro + sp + 3) + u0;
+            const double *pn = src + offB + u0;
 #pragma unroll
             for (int r = 0; r < R; ++r) fpB[r] = pn[lane + 64u * r];
-#pragma unroll
-            for (int j = 0; j < TS; ++j) scB[j] = uload(it + (int64_t)(sp + 3) * SP + j);
         }
+        GDP_SCHED_FENCE();
+        rop += 2;
+        offA = offA2;
+        offB = offB2;
     }
 
 #pragma unroll
@@ -137,7 +177,6 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
         const int s = s0 + j;
         if (s < S) {
             double *drow = dst + (int64_t)s * ld + P + u0;
-            uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (PUBLISH)
@@ -145,7 +184,11 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
                                        __HIP_MEMORY_SCOPE_AGENT);
                 else
                     drow[lane + 64u * r] = best[r][j];
-                mrow[lane + 64u * r] = (uint8_t)arg[r][j];
+            }
+            if constexpr (ARG) {
+                uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
+#pragma unroll
+                for (int r = 0; r < R; ++r) mrow[lane + 64u * r] = (uint8_t)arg[r][j];
             }
         }
     }
@@ -154,7 +197,7 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
 // A tile whose source rows all lie below the first row that can hold a finite cost: every
 // candidate is +inf, so the cell is +inf and its argmin 0 (all-equal candidates go to index 0,
 // csrc/dp_core.cpp:12-16,70).  Same stores as relax_task, no arithmetic.
-template <int TS, int R, bool PUBLISH>
+template <int TS, int R, bool PUBLISH, bool ARG>
 __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
 {
     const int S = uload(&I->S);
@@ -163,7 +206,7 @@ __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsign
     const int64_t ldm = uload(&I->ldm);
     const int nbuf = uload(&I->nbuf);
     double *dst = uload(&I->H) + (int64_t)((layer + 1) % nbuf) * uload(&I->hstride);
-    uint8_t *M = uload(&I->M);
+    [[maybe_unused]] uint8_t *M = uload(&I->M);
     const int s0 = tb * TS;
     const int64_t u0 = (int64_t)tile * (64 * R);
 #pragma unroll
@@ -171,7 +214,6 @@ __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsign
         const int s = s0 + j;
         if (s < S) {
             double *drow = dst + (int64_t)s * ld + P + u0;
-            uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (PUBLISH)
@@ -179,7 +221,11 @@ __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsign
                                        __HIP_MEMORY_SCOPE_AGENT);
                 else
                     drow[lane + 64u * r] = INFINITY;
-                mrow[lane + 64u * r] = 0;
+            }
+            if constexpr (ARG) {
+                uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
+#pragma unroll
+                for (int r = 0; r < R; ++r) mrow[lane + 64u * r] = 0;
             }
         }
     }
@@ -188,22 +234,22 @@ __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsign
 // Rows of a layer that have to be computed (band[3*l+1] .. band[3*l+2], in tiles): below the band
 // every source cell is +inf (fill_task); above it no cell can lie on a path that ends at one of
 // the requested start rows, so nothing is read from there later and nothing is written.
-template <int TS, int R, bool PUBLISH>
+template <int TS, int R, bool PUBLISH, bool ARG>
 __device__ __forceinline__ void tile_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
 {
     const int32_t *band = uload(&I->dep) + 3 * layer;
     const unsigned lo = (unsigned)uload(band + 1), hi = (unsigned)uload(band + 2);
     if (tile > hi) return;
     if (tile < lo)
-        fill_task<TS, R, PUBLISH>(I, layer, tile, tb, lane);
+        fill_task<TS, R, PUBLISH, ARG>(I, layer, tile, tb, lane);
     else
-        relax_task<TS, R, PUBLISH>(I, layer, tile, tb, lane);
+        relax_task<TS, R, PUBLISH, ARG>(I, layer, tile, tb, lane);
 }
 
 // ---- one launch per layer ------------------------------------------------------------------------
 // __launch_bounds__(256, 4): register allocation is held to 4 resident blocks per CU (4 waves per
 // SIMD, at most 128 VGPRs).
-template <int TS, int R>
+template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_kernel(
     const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
 {
@@ -223,13 +269,13 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_kernel(
         const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         if (task >= live_tasks) return;
         const unsigned t = task / ntb;
-        relax_task<TS, R, false>(I, layer, (unsigned)lo + t, task - t * ntb, lane);
+        relax_task<TS, R, false, ARG>(I, layer, (unsigned)lo + t, task - t * ntb, lane);
     } else {
         const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         const unsigned t = task / ntb;
         const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
         if ((int)t > top) return;
-        fill_task<TS, R, false>(I, layer, t, task - t * ntb, lane);
+        fill_task<TS, R, false, ARG>(I, layer, t, task - t * ntb, lane);
     }
 }
 
@@ -270,12 +316,13 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 // One launch for a run of layers (all of them, unless instances of different depth share the
 // batch: then one launch per run of layers with the same set of active instances, so that no
 // launch carries empty workgroups): grid.y = layer - layer0, grid.x = block task (four consecutive
-// (tile, target block) wave tasks of one instance).  Workgroups are dispatched in order of their linear id, x
-// fastest, so every block of layer l is dispatched before any block of layer l+1; a block only
-// ever waits for blocks of the layer before its own, which therefore run or have finished, and the
-// oldest unfinished block never waits: the launch cannot deadlock.  (Each XCD takes every eighth
-// workgroup and dispatches its share in order, which is all the argument needs.)  Older workgroups
-// also win the issue arbitration of their SIMD, so the work that others wait for runs first.
+// (tile, target block) wave tasks of one instance).  Workgroups are dispatched in order of their
+// linear id, x fastest, so every block of layer l is dispatched before any block of layer l+1; a
+// block only ever waits for blocks of the layer before its own, which therefore run or have
+// finished, and the oldest unfinished block never waits: the launch cannot deadlock.  (Each XCD
+// takes every eighth workgroup and dispatches its share in order, which is all the argument needs.)
+// Older workgroups also win the issue arbitration of their SIMD, so the work that others wait for
+// runs first.
 //
 // Instead of a kernel boundary between layers, a task waits only for the tiles it reads: layer l,
 // tile t reads rows of layer l-1's output in tiles [t-dep[l-1], t].  Every layer has its own cost
@@ -289,7 +336,12 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //  - a reader polls the counter with agent-scope loads and only afterwards touches the tile.  Its
 //    L2 cannot hold an older copy of those lines: tiles are whole cache lines, nobody reads a tile
 //    before its counter is full, and the caches are invalidated when the launch begins.
-template <int TS, int R>
+//
+// Share of an XCD: of every instance, one contiguous eighth of the block tasks that carry
+// arithmetic (tiles lo..hi of the layer) and one eighth of the others (tiles below lo are filled
+// with +inf, tiles above hi only counted as done), so that all XCDs carry the same load whatever
+// the bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
+template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_kernel(
     const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q, int layer0)
 {
@@ -299,49 +351,66 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_k
     const int layer = layer0 + (int)blockIdx.y;
     const int max_L = uload(&Q->max_L);
     const int max_ntile = uload(&Q->max_ntile);
-    const int ntb = uload(&Q->ntb);
-    const int nbt = uload(&Q->nbt);
-    const int nat = uload(uload(&Q->n_active) + layer);
-    // The grid is as wide as the fullest layer.  Inside a layer the first `total8` workgroups share
-    // out its block tasks, every XCD getting one contiguous range of them; the rest have nothing to do.
-    const unsigned total = (unsigned)(nat * nbt);
-    const unsigned total8 = (total + 7u) & ~7u;
-    if (blockIdx.x >= total8) return;
-    const unsigned x = xcd_swizzle(blockIdx.x, total8);
-    if (x >= total) return;
-    int32_t *cnt_all = uload(&Q->cnt);
-    int32_t *abort_flag = uload(&Q->abort_flag);
-    const int bt = (int)(x / (unsigned)nat);  // block task within the instance: tiles ascend with x
-    const int ii = (int)x - bt * nat;         // instance (a prefix of the table is active)
+    const unsigned ntb = (unsigned)uload(&Q->ntb);
+    const unsigned nat = (unsigned)uload(uload(&Q->n_active) + layer);
+    const unsigned xcd = blockIdx.x & 7u;   // workgroups go to the XCDs round-robin by linear id;
+    const unsigned pos = blockIdx.x >> 3;   // gridDim.x is a multiple of 8
+    const unsigned w = pos / nat;           // slot within the XCD's share of one instance
+    const unsigned ii = pos - w * nat;      // instance (a prefix of the table is active)
+    if (w >= (unsigned)uload(&Q->slots)) return;
     const GdpDevInst *I = insts + ii;
     const int ntile = uload(&I->ntile);
-    const unsigned q0 = (unsigned)bt * GDP_WAVES_PER_BLOCK;
-    if (layer >= 1) {
+    const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
+    const int32_t *band = uload(&I->dep) + 3 * layer;
+    const int lo = uload(band + 1), hi = uload(band + 2);
+    unsigned bt_lo = 0, n_live = 0;
+    if (hi >= lo) {
+        bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
+        unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
+        if (bt_hi > nbt - 1u) bt_hi = nbt - 1u;
+        n_live = bt_hi - bt_lo + 1u;
+    }
+    const unsigned per_live = (n_live + 7u) >> 3, n_rest = nbt - n_live, per_rest = (n_rest + 7u) >> 3;
+    unsigned bt;
+    bool live;
+    if (w < per_live) {
+        const unsigned i = xcd * per_live + w;
+        if (i >= n_live) return;
+        bt = bt_lo + i;
+        live = true;
+    } else {
+        const unsigned w2 = w - per_live;
+        if (w2 >= per_rest) return;
+        const unsigned i = xcd * per_rest + w2;
+        if (i >= n_rest) return;
+        bt = i < bt_lo ? i : i + n_live;
+        live = false;
+    }
+    int32_t *cnt_all = uload(&Q->cnt);
+    const unsigned q0 = bt * GDP_WAVES_PER_BLOCK;
+    if (live && layer >= 1) {
         // the block's first wave waits for everything its four wave tasks read
         if (wave == 0) {
-            const int t_lo = (int)(q0 / (unsigned)ntb);
-            int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / (unsigned)ntb);
+            const int t_lo = (int)(q0 / ntb);
+            int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / ntb);
             if (t_hi >= ntile) t_hi = ntile - 1;
-            bool ok = true;
-            if (t_lo < ntile) {
-                const int d = uload(uload(&I->dep) + 3 * (layer - 1));
-                const int lo = t_lo - d < 0 ? 0 : t_lo - d;
-                ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, lo, t_hi, ntb, lane,
-                                abort_flag, uload(&Q->spin_limit));
-            }
+            const int d = uload(uload(&I->dep) + 3 * (layer - 1));
+            const int first = t_lo - d < 0 ? 0 : t_lo - d;
+            const bool ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, first, t_hi, (int)ntb,
+                                       lane, uload(&Q->abort_flag), uload(&Q->spin_limit));
             if (lane == 0) sh_ok = ok ? 1 : 0;
         }
         __syncthreads();
         if (__builtin_amdgcn_readfirstlane(sh_ok) == 0) return;  // the launch is being abandoned
     }
     const unsigned q = q0 + wave;
-    const unsigned tile = q / (unsigned)ntb;
-    const unsigned tb = q - tile * (unsigned)ntb;
+    const unsigned tile = q / ntb;
+    const unsigned tb = q - tile * ntb;
     if (tile >= (unsigned)ntile) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // keeps the tile's loads after the wait
-    tile_task<TS, R, true>(I, layer, tile, tb, lane);        // tiles outside the band still count as done
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");    // keeps the tile's loads after the wait
+    tile_task<TS, R, true, ARG>(I, layer, tile, tb, lane);    // tiles outside the band still count as done
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // every write-through store acknowledged
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every write-through store acknowledged
     if (lane == 0)
         __hip_atomic_fetch_add(cnt_all + ((int64_t)ii * max_L + layer) * max_ntile + tile, 1, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
@@ -422,7 +491,12 @@ __device__ __forceinline__ void wave_argmin(double &val, int &idx)
 }
 
 // Epilogue of csrc/dp_core.cpp:78-117 for one key per wavefront: first argmin of the start row,
-// then the dependent walk through the argmin table.
+// then the dependent walk back through the layers.  MARKS: the walk reads the stored argmin table.
+// Otherwise every cost buffer of the run is still there, and the wavefront recomputes the argmin of
+// the one cell per layer that lies on its path, with the arithmetic and the tie-break of the
+// relaxation (csrc/dp_core.cpp:67-73: ascending source strategies, strict '<', so the lowest index
+// among equal candidates, and index 0 when all are +inf).
+template <bool MARKS>
 __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__restrict__ insts,
                                                           const GdpDevKey *__restrict__ keys,
                                                           GdpDevOut *__restrict__ out,
@@ -441,35 +515,67 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
         if (lane == 0) out[blockIdx.x] = o;
         return;
     }
-    const double *fin = uload(&I->H) + (int64_t)(L % uload(&I->nbuf)) * uload(&I->hstride);  // last written
-    const int64_t *ro = uload(&I->roff) + (int64_t)L * (uload(&I->SU) + GDP_SRC_UNROLL);
+    const int nbuf = uload(&I->nbuf);
+    const int64_t hstride = uload(&I->hstride);
+    const double *H = uload(&I->H);
+    const int rows = uload(&I->SU) + GDP_SRC_PAD;
+    const int64_t *roff = uload(&I->roff);
+    const double *fin = H + (int64_t)(L % nbuf) * hstride;  // last written
+    const int64_t *ro = roff + (int64_t)L * rows;
     double val = INFINITY;
     int idx = 0x7fffffff;
     for (int s = lane; s < S; s += 64) {  // ascending within the lane: strict '<' keeps the first
         const double x = fin[ro[s] + v0];
         if (x < val || idx == 0x7fffffff) { val = x; idx = s; }
     }
-    wave_argmin(val, idx);
-    if (lane != 0) return;
+    wave_argmin(val, idx);  // every lane holds the result
+    idx = __builtin_amdgcn_readfirstlane(idx);
     if (!(val < INFINITY)) {  // csrc/dp_core.cpp:93-97
-        out[blockIdx.x] = o;
+        if (lane == 0) out[blockIdx.x] = o;
         return;
     }
     o.total = val + uload(&K->other_time);  // csrc/dp_core.cpp:99
     const int32_t *mem = uload(&I->mem);
-    const uint8_t *M = uload(&I->M);
-    const int64_t ldm = uload(&I->ldm);
     int32_t *path = res + uload(&K->res_off);
     int64_t v = v0;
-    path[L - 1] = idx;
-    for (int i = L - 1; i > 0; --i) {  // csrc/dp_core.cpp:105-113, with mark[i][v][s] = M[i][s][v - mem[i][s]]
-        const int cur = idx;
-        v -= mem[(int64_t)i * S + cur];
-        if (v < 0) break;  // cannot happen on a finite path; keeps a damaged table from being indexed
-        idx = M[((int64_t)i * S + cur) * ldm + v];
-        if (idx >= S) { v = -1; break; }
-        path[i - 1] = idx;
+    if (lane == 0) path[L - 1] = idx;
+    if constexpr (MARKS) {
+        const uint8_t *M = uload(&I->M);
+        const int64_t ldm = uload(&I->ldm);
+        for (int i = L - 1; i > 0; --i) {  // csrc/dp_core.cpp:105-113, with mark[i][v][s] = M[i][s][v - mem[i][s]]
+            const int cur = idx;
+            v -= uload(mem + (int64_t)i * S + cur);
+            if (v < 0) break;  // cannot happen on a finite path; keeps a damaged table from being indexed
+            idx = __builtin_amdgcn_readfirstlane((int)M[((int64_t)i * S + cur) * ldm + v]);
+            if (idx >= S) { v = -1; break; }
+            if (lane == 0) path[i - 1] = idx;
+        }
+    } else {
+        const int SP = uload(&I->SP);
+        const double *inter = uload(&I->inter);
+        const double *intra = uload(&I->intra);
+        const int32_t *inter_index = uload(&I->inter_index);
+        for (int i = L - 1; i > 0; --i) {
+            const int cur = idx;
+            v -= uload(mem + (int64_t)i * S + cur);  // the source row of cell (i, v, cur)
+            if (v < 0) break;
+            const double *src = H + (int64_t)(i % nbuf) * hstride;  // costs before layer i
+            const int64_t *rl = roff + (int64_t)i * rows;
+            const double *it = inter + (int64_t)uload(inter_index + i) * rows * SP + cur;
+            const double a = uload(intra + (int64_t)i * SP + cur);
+            double bv = INFINITY;
+            int bi = 0x7fffffff;
+            for (int s = lane; s < S; s += 64) {
+                const double c = (src[rl[s] + v] + it[(int64_t)s * SP]) + a;
+                if (c < bv || bi == 0x7fffffff) { bv = c; bi = s; }
+            }
+            wave_argmin(bv, bi);
+            idx = __builtin_amdgcn_readfirstlane(bi);
+            if (idx >= S) { v = -1; break; }
+            if (lane == 0) path[i - 1] = idx;
+        }
     }
+    if (lane != 0) return;
     if (v < 0) {
         o.total = INFINITY;
         out[blockIdx.x] = o;
@@ -485,7 +591,7 @@ __global__ __launch_bounds__(256) void gdp_export_f_kernel(const GdpDevInst *__r
 {
     const int L = I->L, V = I->V, S = I->S;
     const double *fin = I->H + (int64_t)(L % I->nbuf) * I->hstride;
-    const int64_t *ro = I->roff + (int64_t)L * (I->SU + GDP_SRC_UNROLL);
+    const int64_t *ro = I->roff + (int64_t)L * (I->SU + GDP_SRC_PAD);
     const int64_t n = (int64_t)V * S;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t v = i / S;
@@ -512,7 +618,7 @@ __global__ __launch_bounds__(256) void gdp_export_mark_kernel(const GdpDevInst *
 
 }  // namespace
 
-template <int TS, int R>
+template <int TS, int R, bool ARG>
 static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_ntile_rows, int SP, int layer,
                                  hipStream_t stream)
 {
@@ -521,18 +627,20 @@ static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_nt
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     nblk = ((nblk + 7u) & ~7u) + 8u;  // live blocks are rounded up to 8, the fill blocks come after them
     dim3 grid(nblk, (unsigned)n_inst, 1), block(64 * GDP_WAVES_PER_BLOCK, 1, 1);
-    hipLaunchKernelGGL((gdp_relax_kernel<TS, R>), grid, block, 0, stream, insts, layer, ntb, nblk);
+    hipLaunchKernelGGL((gdp_relax_kernel<TS, R, ARG>), grid, block, 0, stream, insts, layer, ntb, nblk);
     return hipGetLastError();
 }
 
 // one entry per element of GDP_VARIANTS, in the same order
 #define GDP_FOR_EACH_VARIANT(X) X(0, 8, 4) X(1, 8, 2) X(2, 8, 1) X(3, 11, 3) X(4, 11, 2) X(5, 11, 1)
 
-hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, int max_ntile, int SP, int layer,
-                            hipStream_t stream)
+hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevInst *insts, int n_inst, int max_ntile, int SP,
+                            int layer, hipStream_t stream)
 {
-#define X(id, ts, r) \
-    case id: return launch_relax_t<ts, r>(insts, n_inst, max_ntile, SP, layer, stream);
+#define X(id, ts, r)                                                                                  \
+    case id:                                                                                          \
+        return marks ? launch_relax_t<ts, r, true>(insts, n_inst, max_ntile, SP, layer, stream)       \
+                     : launch_relax_t<ts, r, false>(insts, n_inst, max_ntile, SP, layer, stream);
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
@@ -540,13 +648,16 @@ hipError_t gdp_launch_relax(int variant, const GdpDevInst *insts, int n_inst, in
 #undef X
 }
 
-hipError_t gdp_launch_relax_fused(int variant, const GdpDevInst *insts, const GdpSched *sched, int grid_blocks,
-                                  int layer0, int layers, hipStream_t stream)
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpDevInst *insts, const GdpSched *sched,
+                                  int grid_blocks, int layer0, int layers, hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
-#define X(id, ts, r)                                                                                       \
-    case id:                                                                                               \
-        hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r>), grid, block, 0, stream, insts, sched, layer0); \
+#define X(id, ts, r)                                                                                              \
+    case id:                                                                                                      \
+        if (marks)                                                                                                \
+            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, true>), grid, block, 0, stream, insts, sched, layer0);  \
+        else                                                                                                      \
+            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, false>), grid, block, 0, stream, insts, sched, layer0); \
         break;
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
@@ -576,11 +687,14 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_epilogue(const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,
+hipError_t gdp_launch_epilogue(bool marks, const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,
                                int32_t *res, hipStream_t stream)
 {
     if (n_key <= 0) return hipSuccess;
-    hipLaunchKernelGGL(gdp_epilogue_kernel, dim3((unsigned)n_key), dim3(64), 0, stream, insts, keys, out, res);
+    if (marks)
+        hipLaunchKernelGGL(gdp_epilogue_kernel<true>, dim3((unsigned)n_key), dim3(64), 0, stream, insts, keys, out, res);
+    else
+        hipLaunchKernelGGL(gdp_epilogue_kernel<false>, dim3((unsigned)n_key), dim3(64), 0, stream, insts, keys, out, res);
     return hipGetLastError();
 }
 

@@ -26,6 +26,7 @@ GDP_EXPORT_MARK = 2
 GDP_LAUNCH_FUSED = 4
 GDP_LAUNCH_PER_LAYER = 8
 GDP_COMPUTE_ALL = 16
+GDP_KEEP_MARKS = 32
 GDP_MAX_S = 256
 GDP_OPT_FUSED = 1
 GDP_OPT_SPIN_LIMIT = 2
@@ -122,7 +123,7 @@ class Problem:
 
     def __init__(self, mem, intra, inter, V: int, other_mem: Sequence[int], other_time: Sequence[float], *,
                  inter_index=None, export_f: bool = False, export_mark: bool = False, launch: str | None = None,
-                 compute_all: bool = False):
+                 compute_all: bool = False, keep_marks: bool = False):
         self.mem = np.ascontiguousarray(mem, dtype=np.int32)
         if self.mem.ndim != 2:
             raise ValueError("mem must be [L,S]")
@@ -152,7 +153,7 @@ class Problem:
         self.flags = ((GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0) |
                       (GDP_LAUNCH_FUSED if launch == "fused" else 0) |
                       (GDP_LAUNCH_PER_LAYER if launch == "per_layer" else 0) |
-                      (GDP_COMPUTE_ALL if compute_all else 0))
+                      (GDP_COMPUTE_ALL if compute_all else 0) | (GDP_KEEP_MARKS if keep_marks else 0))
         if self.V < 1 or self.L < 1 or self.S < 1:
             raise ValueError("L, V and S must be >= 1")
         # outputs

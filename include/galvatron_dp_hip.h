@@ -46,8 +46,14 @@ extern "C" {
 #define GDP_EXPORT_F 1u    /* write result.f_out    (final f, reference layout [V][S])       */
 #define GDP_EXPORT_MARK 2u /* write result.mark_out (argmin table, reference layout [L][V][S]) */
 #define GDP_LAUNCH_FUSED 4u     /* lay the plan out for, and use, ONE launch over all layers          */
-#define GDP_LAUNCH_PER_LAYER 8u /* one launch per layer (two cost buffers); default: chosen by size    */
+#define GDP_LAUNCH_PER_LAYER 8u /* one launch per layer; default: chosen by size                          */
 #define GDP_COMPUTE_ALL 16u     /* carry out every one of the L*V*S*S relaxations (see gdp_timing.executed) */
+#define GDP_KEEP_MARKS 32u      /* store the argmin of every cell while relaxing, as the reference does
+                                   (csrc/dp_core.cpp:70-72).  Default: the relaxation computes costs only, the
+                                   cost buffers of all layers stay in device memory, and the backtrack recomputes
+                                   the argmin of the L cells on its path -- same results, two fifths fewer
+                                   instructions.  Implied by GDP_EXPORT_MARK; chosen by the library when the
+                                   per-layer cost buffers do not fit in device memory. */
 
 /* One DP instance == one reference call.  Field <- reference argument (csrc/dp_core.cpp:24-35):
  *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),
@@ -89,7 +95,7 @@ typedef struct gdp_timing {
     double relaxations;    /* sum over instances of L*V*S*S                                    */
     double executed;       /* relaxations actually carried out: cells whose sources are all +inf, and cells
                               that no requested start row can reach back to, are not computed           */
-    double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write) */
+    double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write if kept) */
 } gdp_timing;
 
 typedef struct gdp_plan gdp_plan;
@@ -116,12 +122,11 @@ int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r);
 void gdp_plan_destroy(gdp_plan *plan);
 
 /* Tuning / test knobs of a plan (no counterpart in the reference).
- *   GDP_OPT_FUSED      1 (default): all layers run in ONE launch, every block owns a fixed share of
- *                      the (layer, instance, tile) tasks and waits on per-tile counters;
- *                      0: one launch per layer.  Results are identical.  A plan created with
- *                      GALVATRON_DP_FUSED=0 in the environment, or whose per-layer cost buffers
- *                      did not fit in device memory, keeps two cost buffers and cannot be
- *                      switched to 1.
+ *   GDP_OPT_FUSED      1: all layers run in ONE launch (grid.y = layer), a workgroup waits on the
+ *                      completion counters of the tiles it reads; 0: one launch per layer.  Results
+ *                      are identical; the default is chosen by problem size.  A plan that keeps only
+ *                      two cost buffers (GDP_KEEP_MARKS together with GDP_LAUNCH_PER_LAYER, or per-layer
+ *                      buffers that did not fit in device memory) cannot be switched to 1.
  *   GDP_OPT_SPIN_LIMIT polls a waiting wavefront makes before it gives up; when that happens the
  *                      launch drains normally, the plan switches itself to one launch per layer
  *                      and the run is repeated that way (GDP_E_HIP with GDP_OPT_NO_FALLBACK). */
