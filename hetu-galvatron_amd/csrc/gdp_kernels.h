@@ -36,9 +36,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#ifndef GDP_WAVES_PER_BLOCK
 #define GDP_WAVES_PER_BLOCK 4
-#define GDP_SRC_UNROLL 2  // source strategies are consumed two at a time (padded with +inf sources)
-#define GDP_SRC_PAD 4     // dummy source rows after SU in roff / inter: targets of the last prefetches
+#endif
+#define GDP_SRC_UNROLL 4  // source strategies are consumed up to four per trip (padded with +inf sources)
+#define GDP_SRC_PAD 8     // dummy source rows after SU in roff / inter: targets of the last prefetches
 
 struct GdpDevInst {
     double *H;        // buffer b starts at H + b * hstride

@@ -55,7 +55,14 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const double c = (fp[r] + sc[j]) + add[j];
-            if constexpr (ARG) arg[r][j] = (c < best[r][j]) ? sp : arg[r][j];
+            if constexpr (ARG) {
+                // compare into vcc and select at once: left to the compiler, the compare results of a
+                // whole step end up in as many scalar register pairs, which then spill
+                asm("v_cmp_lt_f64 vcc, %1, %2\n\tv_cndmask_b32 %0, %0, %3, vcc"
+                    : "+v"(arg[r][j])
+                    : "v"(c), "v"(best[r][j]), "v"(sp)
+                    : "vcc");
+            }
             best[r][j] = min_f64(best[r][j], c);
         }
 }
@@ -70,18 +77,9 @@ template <int TS, int R, bool PUBLISH, bool ARG>
 __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb,
                                            unsigned lane)
 {
-    const int S = uload(&I->S);
     const int SU = uload(&I->SU);
     const int SP = uload(&I->SP);
-    const int P = uload(&I->P);
-    const int64_t ld = uload(&I->ld);
-    const int64_t ldm = uload(&I->ldm);
-    const int nbuf = uload(&I->nbuf);
-    const int64_t hstride = uload(&I->hstride);
-    double *const hbase = uload(&I->H);
-    const double *src = hbase + (int64_t)(layer % nbuf) * hstride;
-    double *dst = hbase + (int64_t)((layer + 1) % nbuf) * hstride;
-    [[maybe_unused]] uint8_t *M = uload(&I->M);
+    const double *src = uload(&I->H) + (int64_t)(layer % uload(&I->nbuf)) * uload(&I->hstride);
     const int64_t *ro = uload(&I->roff) + (int64_t)layer * (SU + GDP_SRC_PAD);
     const int s0 = tb * TS;
     const int mat = uload(uload(&I->inter_index) + layer);
@@ -103,75 +101,73 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
             if constexpr (ARG) arg[r][j] = 0;
         }
 
-    // Software pipeline over the source strategies, two per trip (A: even, B: odd), with the order
-    // of issue pinned by scheduling fences, because every load has to be in flight for most of a
-    // half trip (TS*R cells) before its first use:
-    //   - the cost rows of strategy sp+2 are requested as soon as those of sp have been consumed,
-    //     i.e. a whole half trip before they are needed;
-    //   - the transition costs of the next strategy and the row offset of the one after it are
-    //     requested right after the first column of a half trip.  Scalar loads return out of order,
-    //     so waiting for one means waiting for all: after that first column nothing else is pending.
+    // Software pipeline over the source strategies, NS per trip, with the order of issue pinned by
+    // scheduling fences, because a load has to be in flight long before its first use:
+    //   - there are NS register sets of cost rows; the rows of strategy sp+NS are requested as soon
+    //     as those of sp have been consumed, i.e. NS-1 steps (of TS*R cells each) before they are
+    //     needed -- a request that misses the L2 takes several such steps to come back;
+    //   - the transition costs of the next strategy and the row offset for the next request are
+    //     fetched right after the first column of a step.  Scalar loads return out of order, so
+    //     waiting for one means waiting for all: after that first column nothing else is pending.
     // Entries S.. of roff / inter are valid dummies (+inf row, zeros); +inf never wins.
-    double fpA[R], fpB[R], scA[TS], scB[TS];
-    const double *itp = it;                    // row sp of the transition matrix
-    const int64_t *rop = ro;                   // roff[sp]
-    int64_t offA = uload(ro + 2), offB = uload(ro + 3);
+    constexpr int NS = ARG ? 2 : 4;
+    static_assert(GDP_SRC_UNROLL % NS == 0 && NS % 2 == 0 && GDP_SRC_PAD > NS, "padding of roff / inter");
+    double fp[NS][R], sc[2][TS];
+    const double *itp = it;      // row sp of the transition matrix
+    const int64_t *rop = ro;     // roff[sp]
+    int64_t off = uload(ro + NS);
     {
         // same order of issue as inside the loop, so that the waits at the loop head count alike
         // on both ways into it
-        const double *pa = src + uload(ro) + u0;
-        const double *pb = src + uload(ro + 1) + u0;
+        int64_t o0[NS];
+#pragma unroll
+        for (int u = 0; u < NS; ++u) o0[u] = uload(ro + u);
         GDP_SCHED_FENCE();
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            fpA[r] = pa[lane + 64u * r];
-            GDP_SCHED_FENCE();
+        for (int u = 0; u < NS; ++u) {
+            const double *p = src + o0[u] + u0;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                fp[u][r] = p[lane + 64u * r];
+                GDP_SCHED_FENCE();
+            }
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            fpB[r] = pb[lane + 64u * r];
-            GDP_SCHED_FENCE();
-        }
-#pragma unroll
-        for (int j = 0; j < TS; ++j) scA[j] = uload(itp + j);
+        for (int j = 0; j < TS; ++j) sc[0][j] = uload(itp + j);
         GDP_SCHED_FENCE();
     }
-    const int S2 = (S + 1) & ~1;
-    for (int sp = 0; sp < S2; sp += 2) {
-        relax_cols<TS, R, ARG, 0, 1>(best, arg, fpA, scA, add, sp);
-        GDP_SCHED_FENCE();
+    for (int sp = 0; sp < SU; sp += NS) {
 #pragma unroll
-        for (int j = 0; j < TS; ++j) scB[j] = uload(itp + SP + j);
-        const int64_t offA2 = uload(rop + 4);
-        GDP_SCHED_FENCE();
-        relax_cols<TS, R, ARG, 1, TS>(best, arg, fpA, scA, add, sp);
-        GDP_SCHED_FENCE();
-        {
-            const double *pn = src + offA + u0;
+        for (int u = 0; u < NS; ++u) {
+            relax_cols<TS, R, ARG, 0, 1>(best, arg, fp[u], sc[u & 1], add, sp + u);
+            GDP_SCHED_FENCE();
+            itp += SP;
 #pragma unroll
-            for (int r = 0; r < R; ++r) fpA[r] = pn[lane + 64u * r];
+            for (int j = 0; j < TS; ++j) sc[(u + 1) & 1][j] = uload(itp + j);
+            const int64_t off_next = uload(rop + NS + u + 1);
+            GDP_SCHED_FENCE();
+            relax_cols<TS, R, ARG, 1, TS>(best, arg, fp[u], sc[u & 1], add, sp + u);
+            GDP_SCHED_FENCE();
+            {
+                const double *pn = src + off + u0;
+#pragma unroll
+                for (int r = 0; r < R; ++r) fp[u][r] = pn[lane + 64u * r];
+            }
+            GDP_SCHED_FENCE();
+            off = off_next;
         }
-        GDP_SCHED_FENCE();
-        relax_cols<TS, R, ARG, 0, 1>(best, arg, fpB, scB, add, sp + 1);
-        GDP_SCHED_FENCE();
-        itp += 2 * (int64_t)SP;
-#pragma unroll
-        for (int j = 0; j < TS; ++j) scA[j] = uload(itp + j);
-        const int64_t offB2 = uload(rop + 5);
-        GDP_SCHED_FENCE();
-        relax_cols<TS, R, ARG, 1, TS>(best, arg, fpB, scB, add, sp + 1);
-        GDP_SCHED_FENCE();
-        {
-            const double *pn = src + offB + u0;
-#pragma unroll
-            for (int r = 0; r < R; ++r) fpB[r] = pn[lane + 64u * r];
-        }
-        GDP_SCHED_FENCE();
-        rop += 2;
-        offA = offA2;
-        offB = offB2;
+        rop += NS;
     }
 
+    // What the stores need is fetched only now: held in scalar registers across the loop it would
+    // crowd out the loop's own operands.  (The opaque copy keeps the compiler from reusing loads
+    // made before the loop.)
+    const GdpDevInst *J = I;
+    asm volatile("" : "+s"(J));
+    const int S = uload(&J->S);
+    const int P = uload(&J->P);
+    const int64_t ld = uload(&J->ld);
+    double *dst = uload(&J->H) + (int64_t)((layer + 1) % uload(&J->nbuf)) * uload(&J->hstride);
 #pragma unroll
     for (int j = 0; j < TS; ++j) {
         const int s = s0 + j;
@@ -186,7 +182,7 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
                     drow[lane + 64u * r] = best[r][j];
             }
             if constexpr (ARG) {
-                uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
+                uint8_t *mrow = uload(&J->M) + ((int64_t)layer * S + s) * uload(&J->ldm) + u0;
 #pragma unroll
                 for (int r = 0; r < R; ++r) mrow[lane + 64u * r] = (uint8_t)arg[r][j];
             }
@@ -247,10 +243,10 @@ __device__ __forceinline__ void tile_task(const GdpDevInst *I, int layer, unsign
 }
 
 // ---- one launch per layer ------------------------------------------------------------------------
-// __launch_bounds__(256, 4): register allocation is held to 4 resident blocks per CU (4 waves per
-// SIMD, at most 128 VGPRs).
+// __launch_bounds__: register allocation is held to 16 resident waves per CU (4 per SIMD, at most
+// 128 VGPRs).
 template <int TS, int R, bool ARG>
-__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_kernel(
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
     const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
 {
     const GdpDevInst *I = insts + blockIdx.y;
@@ -342,7 +338,7 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 // with +inf, tiles above hi only counted as done), so that all XCDs carry the same load whatever
 // the bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
 template <int TS, int R, bool ARG>
-__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 4) void gdp_relax_fused_kernel(
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
     const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q, int layer0)
 {
     __shared__ int sh_ok;
