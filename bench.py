@@ -18,7 +18,10 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    peak = 39.3 TFLOP/s = MI355X's published 78.6 TFLOP/s fp64 vector rate, which
                    counts an FMA as two operations -- additions and comparisons cannot fuse.
                    ``roofline_hbm`` is the same launch against 8 TB/s with the algorithmic bytes
-                   V*S*(8 read + 8 write + 1 argmin) per layer and instance.
+                   V*S*(8 read + 8 write) per layer and instance (the relaxation stores costs only;
+                   the backtrack recomputes the argmin of the L cells on its path.  ``with_mark_table``
+                   reports the mode that stores the reference's argmin table instead: 17 bytes and
+                   five instead of three vector instructions per relaxation).
 * ``cpu_baseline`` the reference's own dp_core (compiled into oracle/_ref by oracle/build.py) or,
                    where that file is absent, the C restatement in oracle/, timed on this host on a
                    bounded sample of the same workload (its first layers), one thread.
@@ -45,7 +48,7 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 }
 
 
-def _problems(workload: str, compute_all: bool = True):
+def _problems(workload: str, compute_all: bool = True, keep_marks: bool = False):
     from galvatron_dp import _lib, workloads as W
     if workload == "cfg3":
         insts = W.config3()
@@ -56,7 +59,8 @@ def _problems(workload: str, compute_all: bool = True):
         keys = sorted(inst.other_mem)
         probs.append(_lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V,
                                   [inst.other_mem[k] for k in keys], [inst.other_time[k] for k in keys],
-                                  inter_index=inst.inter_index, compute_all=compute_all))
+                                  inter_index=inst.inter_index, compute_all=compute_all,
+                                  keep_marks=keep_marks))
     return insts, probs
 
 
@@ -127,8 +131,8 @@ def main() -> int:
         print(json.dumps({"calibrate_copy_bytes": n, "copies": 3}))
         return 0
 
-    def measure(workload, steps, warmup, compute_all=True):
-        insts, probs = _problems(workload, compute_all)
+    def measure(workload, steps, warmup, compute_all=True, keep_marks=False):
+        insts, probs = _problems(workload, compute_all, keep_marks)
         with _lib.Plan(probs) as plan:
             for _ in range(warmup):
                 plan.run(0)
@@ -165,7 +169,7 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
-                   "mark_bytes": 1, "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
+                   "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
                    "device": _lib.device_info()},
         "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
                      "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,
@@ -190,6 +194,10 @@ def main() -> int:
     line["with_row_skipping"] = {"value_nominal": ms["value"], "ms_per_step": ms["ms_per_step"],
                                  "relaxations_executed_fraction": ms["executed_fraction"],
                                  "roofline_frac_valu_fp64_executed": ms["tflops"] / PEAK_FP64_VALU_TFLOPS}
+    mk = measure(a.workload, max(3, a.steps // 2), 1, keep_marks=True)
+    line["with_mark_table"] = {"value": mk["value"], "ms_per_step": mk["ms_per_step"],
+                               "roofline_frac_valu_fp64": mk["tflops"] / PEAK_FP64_VALU_TFLOPS,
+                               "algorithmic_bytes_per_launch": mk["bytes_per_launch"]}
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(a.workload)
     print(json.dumps(line))

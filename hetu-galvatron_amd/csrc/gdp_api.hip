@@ -337,13 +337,22 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
     }
     if (!fused_preset) {
-        // One launch for all layers pays off when a layer holds at least twice as many block tasks as
-        // the device holds blocks: then what a block waits for was finished a while ago, and its
-        // loads, stores and waits hide under the arithmetic of its neighbours.  Below that the
-        // latency of signalling through memory shows, and a launch per layer is quicker.
-        int64_t first_layer = 0;
-        for (const Group &g : pl->groups) first_layer += (int64_t)g.active[0] * g.nbt;
-        pl->fused = first_layer >= 2 * (int64_t)pl->num_cu * 4;
+        // One launch for all layers pays off when a layer holds at least twice as many block tasks
+        // that carry arithmetic as the device holds blocks: then what a block waits for was finished a
+        // while ago, and its loads, stores and waits hide under the arithmetic of its neighbours.
+        // Below that the latency of signalling through memory shows, and a launch per layer is quicker.
+        double first_layer = 0, all = 0, live = 0;
+        std::vector<int32_t> band;
+        for (const Group &g : pl->groups) {
+            first_layer += (double)g.active[0] * g.nbt;
+            for (int k = g.first; k < g.first + g.count; ++k) {
+                const HostInst &h = inst[(size_t)k];
+                band.assign((size_t)h.L * 3, 0);
+                fill_bands(p[h.orig], h, 64 * GDP_VARIANTS[h.variant].r, pl->skip, band.data(), &live);
+                all += (double)h.L * h.V * (double)h.S * h.S;
+            }
+        }
+        pl->fused = first_layer * (all > 0 ? live / all : 1.0) >= 2.0 * pl->num_cu * 4;
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -485,7 +494,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
         sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb;
-        sc->slots = (g.nbt + 7) / 8 + 1;
+        sc->slots = (g.nbt + 7) / 8 + 2;
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
         for (int l = 0; l < g.max_L; ++l) act[l] = g.active[(size_t)l];
@@ -552,8 +561,8 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                                 pl->stream));
         for (const Group &g : pl->groups)
             for (const auto &seg : g.segments) {  // (first layer, number of layers)
-                // per XCD and instance: an eighth of the block tasks inside the band and an eighth of the rest
-                const int grid_x = 8 * g.active[(size_t)seg.first] * ((g.nbt + 7) / 8 + 1);
+                // per XCD and instance: an eighth each of the block tasks below, inside and above the band
+                const int grid_x = 8 * g.active[(size_t)seg.first] * ((g.nbt + 7) / 8 + 2);
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
                 GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks, d_insts + g.first,
                                                reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,

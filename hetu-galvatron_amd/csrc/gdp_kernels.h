@@ -68,7 +68,7 @@ struct GdpSched {
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
     int32_t max_L, max_ntile, ntb;
-    int32_t slots;            // workgroups per XCD, instance and layer: ceil(block tasks / 8) + 1
+    int32_t slots;            // workgroups per XCD, instance and layer: ceil(block tasks / 8) + 2
     int64_t spin_limit;       // polls before a waiting wave gives up
 };
 

@@ -334,9 +334,9 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //    before its counter is full, and the caches are invalidated when the launch begins.
 //
 // Share of an XCD: of every instance, one contiguous eighth of the block tasks that carry
-// arithmetic (tiles lo..hi of the layer) and one eighth of the others (tiles below lo are filled
-// with +inf, tiles above hi only counted as done), so that all XCDs carry the same load whatever
-// the bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
+// arithmetic (tiles lo..hi of the layer), one eighth of those below (filled with +inf) and one
+// eighth of those above (only counted as done), so that all XCDs carry the same load whatever the
+// bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
 template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
     const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q, int layer0)
@@ -366,21 +366,29 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         if (bt_hi > nbt - 1u) bt_hi = nbt - 1u;
         n_live = bt_hi - bt_lo + 1u;
     }
-    const unsigned per_live = (n_live + 7u) >> 3, n_rest = nbt - n_live, per_rest = (n_rest + 7u) >> 3;
+    // Order inside the XCD's share of an instance: the block tasks below the band first (they only
+    // store +inf, and the layer after this one waits for some of them), then the ones that carry
+    // arithmetic, then those above the band (nothing to do but to count as done).
+    const unsigned n_fill = bt_lo, n_dead = nbt - n_fill - n_live;
+    const unsigned per_fill = (n_fill + 7u) >> 3, per_live = (n_live + 7u) >> 3, per_dead = (n_dead + 7u) >> 3;
     unsigned bt;
-    bool live;
-    if (w < per_live) {
-        const unsigned i = xcd * per_live + w;
+    bool live = false;
+    if (w < per_fill) {
+        const unsigned i = xcd * per_fill + w;
+        if (i >= n_fill) return;
+        bt = n_fill - 1u - i;  // from the band downwards: the lowest tiles of the next layer's band, which
+                               // XCD 0 computes, read the tiles just below this layer's band
+    } else if (w < per_fill + per_live) {
+        const unsigned i = xcd * per_live + (w - per_fill);
         if (i >= n_live) return;
         bt = bt_lo + i;
         live = true;
     } else {
-        const unsigned w2 = w - per_live;
-        if (w2 >= per_rest) return;
-        const unsigned i = xcd * per_rest + w2;
-        if (i >= n_rest) return;
-        bt = i < bt_lo ? i : i + n_live;
-        live = false;
+        const unsigned w2 = w - per_fill - per_live;
+        if (w2 >= per_dead) return;
+        const unsigned i = xcd * per_dead + w2;
+        if (i >= n_dead) return;
+        bt = bt_lo + n_live + i;
     }
     int32_t *cnt_all = uload(&Q->cnt);
     const unsigned q0 = bt * GDP_WAVES_PER_BLOCK;

@@ -1,5 +1,7 @@
 """GPU tests of the batched entry points and of the two launch schemes (one launch per layer /
 one launch for all layers), through the C ABI."""
+import os
+
 import numpy as np
 import pytest
 
@@ -85,6 +87,27 @@ def test_skipping_rows_changes_nothing(golden, name, launch):
     prob = _problem(inst, launch=launch, export_f=True, export_mark=True)
     _lib.solve_batch([prob])
     assert H.sha(prob.f_out) == rec["f_sha256"] and H.sha(prob.mark_out) == rec["mark_sha256"]
+
+
+@pytest.mark.parametrize("launch", ["fused", "per_layer"])
+@pytest.mark.parametrize("keep_marks", [False, True])
+@pytest.mark.parametrize("name", ["cfg2_small", "cfg4_small", "galvatron_like", "ties_3", "infeasible_6",
+                                  "cfg3_smallV_2"])
+def test_costs_only_and_mark_table_modes_agree(golden, name, launch, keep_marks):
+    """Default: the relaxation stores costs only and the backtrack recomputes the argmin of the cells
+    on its path.  keep_marks: the argmin table is stored as in the reference.  Same results, same f."""
+    rec = golden[name]
+    inst = H.build_case(rec)
+    prob = _problem(inst, launch=launch, keep_marks=keep_marks, export_f=True)
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)
+        t = plan.run(1)
+        plan.fetch()
+    _check_against_golden(prob, rec, f"{name} keep_marks={keep_marks}")
+    assert H.sha(prob.f_out) == rec["f_sha256"]
+    if "GALVATRON_DP_KEEP_MARKS" not in os.environ:     # a preset in the environment overrides the flag
+        cells = float(inst.L) * inst.V * inst.S
+        assert t.relax_bytes == cells * (17 if keep_marks else 16)
 
 
 def test_abandoned_fused_launch_falls_back_or_reports(golden):

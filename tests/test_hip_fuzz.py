@@ -19,22 +19,27 @@ SHAPES = [(1, 1, 1), (1, 1, 7), (2, 1, 64), (3, 2, 65), (4, 7, 191), (3, 8, 192)
 
 
 def _compare(inst, tag, launch=None):
+    """Two solves of the same instance: costs-only relaxation with the argmin recomputed on the
+    backtrack (the default; f exported, which does not change the mode) and the mode that keeps
+    the reference's mark table (forced by exporting it)."""
     keys = sorted(inst.other_mem)
-    prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
-                        [inst.other_time[k] for k in keys], inter_index=inst.inter_index, export_f=True,
-                        export_mark=True, launch=launch)
-    with _lib.Plan([prob]) as plan:
-        plan.set_option(_lib.GDP_OPT_POISON, 1)
-        plan.run()
-        plan.fetch()
     wt, wr, wm, wf, wmark = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time,
                                     keep=True)
-    got = ({k: prob.total[i] for i, k in enumerate(keys)},
-           {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
-           {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
-    H.assert_same_results(got, (wt, wr, wm), tag)
-    assert prob.f_out.tobytes() == wf.tobytes(), f"{tag}: f differs"
-    assert np.array_equal(prob.mark_out, wmark), f"{tag}: mark differs"
+    for marks in (False, True):
+        prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                            [inst.other_time[k] for k in keys], inter_index=inst.inter_index, export_f=True,
+                            export_mark=marks, launch=launch)
+        with _lib.Plan([prob]) as plan:
+            plan.set_option(_lib.GDP_OPT_POISON, 1)
+            plan.run()
+            plan.fetch()
+        got = ({k: prob.total[i] for i, k in enumerate(keys)},
+               {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+               {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+        H.assert_same_results(got, (wt, wr, wm), f"{tag} marks={marks}")
+        assert prob.f_out.tobytes() == wf.tobytes(), f"{tag} marks={marks}: f differs"
+        if marks:
+            assert np.array_equal(prob.mark_out, wmark), f"{tag}: mark differs"
 
 
 @pytest.mark.parametrize("n,shape", list(enumerate(SHAPES)))
