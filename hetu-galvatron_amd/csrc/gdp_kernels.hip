@@ -351,9 +351,13 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned nat = (unsigned)uload(uload(&Q->n_active) + layer);
     const unsigned xcd = blockIdx.x & 7u;   // workgroups go to the XCDs round-robin by linear id;
     const unsigned pos = blockIdx.x >> 3;   // gridDim.x is a multiple of 8
-    const unsigned w = pos / nat;           // slot within the XCD's share of one instance
-    const unsigned ii = pos - w * nat;      // instance (a prefix of the table is active)
-    if (w >= (unsigned)uload(&Q->slots)) return;
+    // Instance-major: the workgroups that an XCD runs at the same time work on neighbouring tiles of
+    // a few instances, whose source rows overlap (a tile reads dep+1 tiles of the layer before), so
+    // that the overlap is fetched from HBM once and then found in this XCD's L2.
+    const unsigned slots = (unsigned)uload(&Q->slots);
+    const unsigned ii = pos / slots;        // instance (a prefix of the table is active)
+    const unsigned w = pos - ii * slots;    // slot within the XCD's share of that instance
+    if (ii >= nat) return;
     const GdpDevInst *I = insts + ii;
     const int ntile = uload(&I->ntile);
     const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
