@@ -47,7 +47,7 @@ struct HostInst {
     int key_begin;  // first entry in the key table
     int res_begin;  // first element in the result array
     // byte offsets inside the device allocation
-    size_t off_H, off_M, off_inter, off_intra, off_index, off_roff, off_mem, off_dep;
+    size_t off_H, off_M, off_inter, off_intra, off_index, off_roff, off_mem;
 };
 
 struct Group {  // instances with the same S, sorted by L descending
@@ -55,7 +55,7 @@ struct Group {  // instances with the same S, sorted by L descending
     int64_t max_ld;
     std::vector<int> active;  // active[l] = number of instances with L > l
     std::vector<std::pair<int, int>> segments;  // fused launches: (first layer, layers), same active set
-    size_t off_sched, off_active, off_cnt;  // byte offsets in the device allocation
+    size_t off_sched, off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
 // Target-tile width: the one that pads S the least (ties: the first).
@@ -374,6 +374,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     for (auto &g : pl->groups) {
         g.off_sched = take(sizeof(GdpSched));
         g.off_active = take(sizeof(int32_t) * (size_t)g.max_L);
+        g.off_lay = take(sizeof(GdpDevLayer) * (size_t)g.count * (size_t)g.max_L);
     }
     for (auto &h : inst) {
         h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_PAD) * h.SP);
@@ -381,7 +382,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
         h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_PAD));
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
-        h.off_dep = take(sizeof(int32_t) * (size_t)h.L * 3);
     }
     const size_t small_bytes = off;
     // words that every run resets to zero: abort flag, ticket counters, completion counters
@@ -428,6 +428,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     } catch (const std::bad_alloc &) {
         return fail(GDP_E_NOMEM, "host staging allocation failed");
     }
+    std::vector<std::vector<int32_t>> h_band((size_t)n);
     GdpDevInst *di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
     GdpDevKey *dk = reinterpret_cast<GdpDevKey *>(stage.data() + pl->off_keys);
     for (int i = 0; i < n; ++i) {
@@ -443,7 +444,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         d.inter_index = reinterpret_cast<const int32_t *>(pl->dbase + h.off_index);
         d.roff = reinterpret_cast<const int64_t *>(pl->dbase + h.off_roff);
         d.mem = reinterpret_cast<const int32_t *>(pl->dbase + h.off_mem);
-        d.dep = reinterpret_cast<const int32_t *>(pl->dbase + h.off_dep);
         d.ld = h.ld; d.ldm = h.ldm;
         d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.SU = h.SU; d.P = h.P; d.ntile = h.ntile;
         const int rows = h.SU + GDP_SRC_PAD;  // source rows per matrix / offsets per layer
@@ -475,9 +475,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
             }
             for (int s = h.S; s < rows; ++s) row[s] = inf_row;  // padding sources and prefetch targets
         }
-        // dep[l] = {tiles a reader reaches down, first tile to compute, last tile to compute}
-        int32_t *dep = reinterpret_cast<int32_t *>(stage.data() + h.off_dep);
-        fill_bands(q, h, tile_rows, pl->skip, dep, &pl->executed);
+        // {tiles a reader reaches down, first tile to compute, last tile to compute} per layer
+        h_band[(size_t)i].assign((size_t)h.L * 3, 0);
+        fill_bands(q, h, tile_rows, pl->skip, h_band[(size_t)i].data(), &pl->executed);
         for (int k = 0; k < h.n_key; ++k) {
             GdpDevKey &key = dk[h.key_begin + k];
             key.other_mem = q->other_mem[k];
@@ -490,6 +490,32 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     }
     for (auto &g : pl->groups) {
         GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
+        // the per-(instance, layer) records; entries of layers an instance does not have stay zero but for hi
+        GdpDevLayer *lay = reinterpret_cast<GdpDevLayer *>(stage.data() + g.off_lay);
+        sc->lay = reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay);
+        for (int k = 0; k < g.count; ++k) {
+            const HostInst &h = inst[(size_t)(g.first + k)];
+            const gdp_problem *q = p[h.orig];
+            const GdpDevInst &d = di[g.first + k];
+            const int rows = h.SU + GDP_SRC_PAD;
+            for (int l = 0; l < g.max_L; ++l) {
+                GdpDevLayer &y = lay[(size_t)k * g.max_L + l];
+                y.hi = -1;
+                if (l >= h.L) continue;
+                const int mat = q->inter_index ? q->inter_index[l] : l;
+                y.src = d.H + (int64_t)(l % h.nbuf) * d.hstride;
+                y.dst = d.H + (int64_t)((l + 1) % h.nbuf) * d.hstride + h.P;
+                y.ro = d.roff + (int64_t)l * rows;
+                y.it = d.inter + (int64_t)mat * rows * h.SP;
+                y.ia = d.intra + (int64_t)l * h.SP;
+                y.m = d.M ? d.M + (int64_t)l * h.S * h.ldm : nullptr;
+                y.ld = h.ld; y.ldm = h.ldm;
+                y.S = h.S; y.SU = h.SU; y.SP = h.SP; y.ntile = h.ntile;
+                y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
+                y.lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
+                y.hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
+            }
+        }
         sc->cnt = reinterpret_cast<int32_t *>(pl->dbase + g.off_cnt);
         sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
@@ -564,7 +590,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                 // per XCD and instance: an eighth each of the block tasks below, inside and above the band
                 const int grid_x = 8 * g.active[(size_t)seg.first] * ((g.nbt + 7) / 8 + 2);
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks, d_insts + g.first,
+                GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
                                                reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,
                                                seg.first, seg.second, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
@@ -575,8 +601,9 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
             for (const Group &g : pl->groups) {
                 if (l >= g.max_L) continue;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, d_insts + g.first, g.active[(size_t)l], g.max_ntile,
-                                         g.SP, l, pl->stream));
+                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks,
+                                         reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
+                                         g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }

@@ -25,13 +25,17 @@
 //          padded with zeros up to SP = a multiple of the target tile).
 //   intra  L rows of SP doubles (zero padded).
 //   mem    L rows of S int32, as given.
-//   dep    L rows of 3 int32: {dep, lo, hi}.  dep = ceil(max mem[l] / tile rows): a reader of layer
-//          l's output at tile t touches tiles [t-dep, t].  lo/hi: the band of tiles of layer l that
-//          has to be computed.  Source rows below sum_{k<l} min_s mem[k][s] hold only +inf, so tiles
-//          entirely below are filled with +inf / argmin 0 without arithmetic (bit-identical to
-//          computing them).  Source rows above max start row - sum_{k>=l} min_s mem[k][s] cannot lie
-//          on any path that ends at a requested start row; they are skipped unless the caller asked
-//          for the full f / mark arrays.
+//
+// The relaxation kernels do not read the instance record at all: everything one (instance, layer)
+// step needs is precomputed into one 128-byte GdpDevLayer record (one scalar load away from the
+// kernel arguments), in a table of n_inst x max_L records per group of instances.
+//   dep    ceil(max mem[l] / tile rows): a reader of layer l's output at tile t touches tiles
+//          [t-dep, t].
+//   lo/hi  the band of tiles of layer l that has to be computed.  Source rows below
+//          sum_{k<l} min_s mem[k][s] hold only +inf, so tiles entirely below are filled with
+//          +inf / argmin 0 without arithmetic (bit-identical to computing them).  Source rows above
+//          max start row - sum_{k>=l} min_s mem[k][s] cannot lie on any path that ends at a
+//          requested start row; they are skipped unless the caller asked for the full f / mark arrays.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -51,8 +55,6 @@ struct GdpDevInst {
     const int32_t *inter_index;
     const int64_t *roff;
     const int32_t *mem;
-    const int32_t *dep;  // [L][3]: tiles below a tile that a reader of layer l's output needs; first and
-                         // last tile of layer l that has to be computed (see tile_task)
     int64_t ld;          // elements per row of H
     int64_t ldm;         // entries per row of M
     int32_t L, V, S, SP;
@@ -62,8 +64,24 @@ struct GdpDevInst {
     int32_t nbuf;
 };
 
+// One relaxation step of one instance, ready to use.
+struct GdpDevLayer {
+    const double *src;  // cost buffer this layer reads; roff offsets are relative to it
+    double *dst;        // row 0, source row 0 (element P) of the cost buffer this layer writes
+    const int64_t *ro;  // this layer's row of roff
+    const double *it;   // this layer's transition matrix
+    const double *ia;   // this layer's row of intra
+    uint8_t *m;         // this layer's S rows of the argmin table (null when marks are not kept)
+    int64_t ld, ldm;    // elements per row of H / entries per row of M
+    int32_t S, SU, SP, ntile;
+    int32_t dep, lo, hi;  // see above; an entry of an instance without this layer has lo = 0, hi = -1
+    int32_t pad_[9];
+};
+static_assert(sizeof(GdpDevLayer) == 128, "one record = two 64-byte scalar loads");
+
 // Bookkeeping of one fused (all layers) launch over a group of instances.
 struct GdpSched {
+    const GdpDevLayer *lay;   // [n_inst][max_L]
     int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
@@ -94,13 +112,14 @@ static const GdpVariant GDP_VARIANTS[] = {{8, 4}, {8, 2}, {8, 1}, {11, 3}, {11, 
 #define GDP_NUM_VARIANTS 6
 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
-// marks: track and store the argmin table (otherwise costs only).
-hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevInst *insts, int n_inst, int max_ntile, int SP,
-                            int layer, hipStream_t stream);
+// marks: track and store the argmin table (otherwise costs only).  lay: the group's table of
+// n_inst x max_L records.
+hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile,
+                            int SP, int layer, hipStream_t stream);
 // Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpDevInst *insts, const GdpSched *sched,
-                                  int grid_blocks, int layer0, int layers, hipStream_t stream);
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
+                                  int layers, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
 // in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).

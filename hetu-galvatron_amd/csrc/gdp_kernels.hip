@@ -67,24 +67,23 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
         }
 }
 
-// One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of layer `layer`.
+// One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of the layer described
+// by Y.
 // PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
 // waits for this task's completion counter finds them in memory.
 // ARG: also track and store the argmin (the reference's mark table, csrc/dp_core.cpp:70-72).  Without
 // it a relaxation is two additions and one minimum; the backtrack then recomputes the argmin of the
 // few cells on its path from the cost buffers, all of which are kept in that mode.
 template <int TS, int R, bool PUBLISH, bool ARG>
-__device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb,
-                                           unsigned lane)
+__device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
 {
-    const int SU = uload(&I->SU);
-    const int SP = uload(&I->SP);
-    const double *src = uload(&I->H) + (int64_t)(layer % uload(&I->nbuf)) * uload(&I->hstride);
-    const int64_t *ro = uload(&I->roff) + (int64_t)layer * (SU + GDP_SRC_PAD);
+    const int SU = uload(&Y->SU);
+    const int SP = uload(&Y->SP);
+    const double *src = uload(&Y->src);
+    const int64_t *ro = uload(&Y->ro);
     const int s0 = tb * TS;
-    const int mat = uload(uload(&I->inter_index) + layer);
-    const double *it = uload(&I->inter) + (int64_t)mat * (SU + GDP_SRC_PAD) * SP + s0;
-    const double *ia = uload(&I->intra) + (int64_t)layer * SP + s0;
+    const double *it = uload(&Y->it) + s0;
+    const double *ia = uload(&Y->ia) + s0;
     const int64_t u0 = (int64_t)tile * (64 * R);
 
     double add[TS];
@@ -162,17 +161,20 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
     // What the stores need is fetched only now: held in scalar registers across the loop it would
     // crowd out the loop's own operands.  (The opaque copy keeps the compiler from reusing loads
     // made before the loop.)
-    const GdpDevInst *J = I;
-    asm volatile("" : "+s"(J));
-    const int S = uload(&J->S);
-    const int P = uload(&J->P);
-    const int64_t ld = uload(&J->ld);
-    double *dst = uload(&J->H) + (int64_t)((layer + 1) % uload(&J->nbuf)) * uload(&J->hstride);
+    const GdpDevLayer *Z = Y;
+    asm volatile("" : "+s"(Z));
+    const int64_t ld = uload(&Z->ld);
+    const int nvalid = uload(&Z->S) - s0;  // target strategies of this block that exist (>= 1)
+    double *drow = uload(&Z->dst) + (int64_t)s0 * ld + u0;
+    [[maybe_unused]] uint8_t *mrow = nullptr;
+    [[maybe_unused]] int64_t ldm = 0;
+    if constexpr (ARG) {
+        ldm = uload(&Z->ldm);
+        mrow = uload(&Z->m) + (int64_t)s0 * ldm + u0;
+    }
 #pragma unroll
     for (int j = 0; j < TS; ++j) {
-        const int s = s0 + j;
-        if (s < S) {
-            double *drow = dst + (int64_t)s * ld + P + u0;
+        if (j < nvalid) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (PUBLISH)
@@ -182,10 +184,11 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
                     drow[lane + 64u * r] = best[r][j];
             }
             if constexpr (ARG) {
-                uint8_t *mrow = uload(&J->M) + ((int64_t)layer * S + s) * uload(&J->ldm) + u0;
 #pragma unroll
                 for (int r = 0; r < R; ++r) mrow[lane + 64u * r] = (uint8_t)arg[r][j];
+                mrow += ldm;
             }
+            drow += ld;
         }
     }
 }
@@ -194,22 +197,22 @@ __device__ __forceinline__ void relax_task(const GdpDevInst *I, int layer, unsig
 // candidate is +inf, so the cell is +inf and its argmin 0 (all-equal candidates go to index 0,
 // csrc/dp_core.cpp:12-16,70).  Same stores as relax_task, no arithmetic.
 template <int TS, int R, bool PUBLISH, bool ARG>
-__device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
+__device__ __forceinline__ void fill_task(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
 {
-    const int S = uload(&I->S);
-    const int P = uload(&I->P);
-    const int64_t ld = uload(&I->ld);
-    const int64_t ldm = uload(&I->ldm);
-    const int nbuf = uload(&I->nbuf);
-    double *dst = uload(&I->H) + (int64_t)((layer + 1) % nbuf) * uload(&I->hstride);
-    [[maybe_unused]] uint8_t *M = uload(&I->M);
     const int s0 = tb * TS;
     const int64_t u0 = (int64_t)tile * (64 * R);
+    const int64_t ld = uload(&Y->ld);
+    const int nvalid = uload(&Y->S) - s0;
+    double *drow = uload(&Y->dst) + (int64_t)s0 * ld + u0;
+    [[maybe_unused]] uint8_t *mrow = nullptr;
+    [[maybe_unused]] int64_t ldm = 0;
+    if constexpr (ARG) {
+        ldm = uload(&Y->ldm);
+        mrow = uload(&Y->m) + (int64_t)s0 * ldm + u0;
+    }
 #pragma unroll
     for (int j = 0; j < TS; ++j) {
-        const int s = s0 + j;
-        if (s < S) {
-            double *drow = dst + (int64_t)s * ld + P + u0;
+        if (j < nvalid) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (PUBLISH)
@@ -219,27 +222,27 @@ __device__ __forceinline__ void fill_task(const GdpDevInst *I, int layer, unsign
                     drow[lane + 64u * r] = INFINITY;
             }
             if constexpr (ARG) {
-                uint8_t *mrow = M + ((int64_t)layer * S + s) * ldm + u0;
 #pragma unroll
                 for (int r = 0; r < R; ++r) mrow[lane + 64u * r] = 0;
+                mrow += ldm;
             }
+            drow += ld;
         }
     }
 }
 
-// Rows of a layer that have to be computed (band[3*l+1] .. band[3*l+2], in tiles): below the band
-// every source cell is +inf (fill_task); above it no cell can lie on a path that ends at one of
-// the requested start rows, so nothing is read from there later and nothing is written.
+// Rows of a layer that have to be computed (tiles lo .. hi): below the band every source cell is
+// +inf (fill_task); above it no cell can lie on a path that ends at one of the requested start
+// rows, so nothing is read from there later and nothing is written.
 template <int TS, int R, bool PUBLISH, bool ARG>
-__device__ __forceinline__ void tile_task(const GdpDevInst *I, int layer, unsigned tile, unsigned tb, unsigned lane)
+__device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, unsigned tile, unsigned tb,
+                                          unsigned lane)
 {
-    const int32_t *band = uload(&I->dep) + 3 * layer;
-    const unsigned lo = (unsigned)uload(band + 1), hi = (unsigned)uload(band + 2);
-    if (tile > hi) return;
-    if (tile < lo)
-        fill_task<TS, R, PUBLISH, ARG>(I, layer, tile, tb, lane);
+    if ((int)tile > hi) return;
+    if ((int)tile < lo)
+        fill_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
     else
-        relax_task<TS, R, PUBLISH, ARG>(I, layer, tile, tb, lane);
+        relax_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
 }
 
 // ---- one launch per layer ------------------------------------------------------------------------
@@ -247,31 +250,29 @@ __device__ __forceinline__ void tile_task(const GdpDevInst *I, int layer, unsign
 // 128 VGPRs).
 template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
-    const GdpDevInst *__restrict__ insts, int layer, unsigned ntb, unsigned nblk_x)
+    const GdpDevLayer *__restrict__ lay, int max_L, int layer, unsigned ntb)
 {
-    const GdpDevInst *I = insts + blockIdx.y;
-    if (layer >= uload(&I->L)) return;
+    const GdpDevLayer *Y = lay + ((int64_t)blockIdx.y * max_L + layer);
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned lane = threadIdx.x & 63u;
     // Only the tiles lo..hi of this layer carry arithmetic.  The first blocks of the grid share them
     // out, every XCD getting one contiguous range of them (equal work per XCD, neighbouring budget
     // rows in one L2); the blocks after those fill the tiles below lo; tiles above hi are left alone.
-    const int32_t *band = uload(&I->dep) + 3 * layer;
-    const int lo = uload(band + 1), hi = uload(band + 2);
+    // (A table entry of an instance that has no such layer has hi = -1 and lo = 0.)
+    const int lo = uload(&Y->lo), hi = uload(&Y->hi);
     const unsigned live_tasks = hi >= lo ? (unsigned)(hi - lo + 1) * ntb : 0u;
     const unsigned live_blocks = ((live_tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK + 7u) & ~7u;
-    (void)nblk_x;
     if (blockIdx.x < live_blocks) {
         const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         if (task >= live_tasks) return;
         const unsigned t = task / ntb;
-        relax_task<TS, R, false, ARG>(I, layer, (unsigned)lo + t, task - t * ntb, lane);
+        relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
     } else {
         const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         const unsigned t = task / ntb;
         const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
         if ((int)t > top) return;
-        fill_task<TS, R, false, ARG>(I, layer, t, task - t * ntb, lane);
+        fill_task<TS, R, false, ARG>(Y, t, task - t * ntb, lane);
     }
 }
 
@@ -339,7 +340,7 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 // bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
 template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
-    const GdpDevInst *__restrict__ insts, const GdpSched *__restrict__ Q, int layer0)
+    const GdpSched *__restrict__ Q, int layer0)
 {
     __shared__ int sh_ok;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -358,11 +359,10 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned ii = pos / slots;        // instance (a prefix of the table is active)
     const unsigned w = pos - ii * slots;    // slot within the XCD's share of that instance
     if (ii >= nat) return;
-    const GdpDevInst *I = insts + ii;
-    const int ntile = uload(&I->ntile);
+    const GdpDevLayer *Y = uload(&Q->lay) + ((int64_t)ii * max_L + layer);
+    const int ntile = uload(&Y->ntile);
     const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
-    const int32_t *band = uload(&I->dep) + 3 * layer;
-    const int lo = uload(band + 1), hi = uload(band + 2);
+    const int lo = uload(&Y->lo), hi = uload(&Y->hi);
     unsigned bt_lo = 0, n_live = 0;
     if (hi >= lo) {
         bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
             const int t_lo = (int)(q0 / ntb);
             int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / ntb);
             if (t_hi >= ntile) t_hi = ntile - 1;
-            const int d = uload(uload(&I->dep) + 3 * (layer - 1));
+            const int d = uload(&Y[-1].dep);
             const int first = t_lo - d < 0 ? 0 : t_lo - d;
             const bool ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, first, t_hi, (int)ntb,
                                        lane, uload(&Q->abort_flag), uload(&Q->spin_limit));
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned tb = q - tile * ntb;
     if (tile >= (unsigned)ntile) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");    // keeps the tile's loads after the wait
-    tile_task<TS, R, true, ARG>(I, layer, tile, tb, lane);    // tiles outside the band still count as done
+    tile_task<TS, R, true, ARG>(Y, lo, hi, tile, tb, lane);   // tiles outside the band still count as done
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every write-through store acknowledged
     if (lane == 0)
@@ -627,7 +627,7 @@ __global__ __launch_bounds__(256) void gdp_export_mark_kernel(const GdpDevInst *
 }  // namespace
 
 template <int TS, int R, bool ARG>
-static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_ntile_rows, int SP, int layer,
+static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile_rows, int SP, int layer,
                                  hipStream_t stream)
 {
     const unsigned ntb = (unsigned)(SP / TS);
@@ -635,20 +635,20 @@ static hipError_t launch_relax_t(const GdpDevInst *insts, int n_inst, int max_nt
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     nblk = ((nblk + 7u) & ~7u) + 8u;  // live blocks are rounded up to 8, the fill blocks come after them
     dim3 grid(nblk, (unsigned)n_inst, 1), block(64 * GDP_WAVES_PER_BLOCK, 1, 1);
-    hipLaunchKernelGGL((gdp_relax_kernel<TS, R, ARG>), grid, block, 0, stream, insts, layer, ntb, nblk);
+    hipLaunchKernelGGL((gdp_relax_kernel<TS, R, ARG>), grid, block, 0, stream, lay, max_L, layer, ntb);
     return hipGetLastError();
 }
 
 // one entry per element of GDP_VARIANTS, in the same order
 #define GDP_FOR_EACH_VARIANT(X) X(0, 8, 4) X(1, 8, 2) X(2, 8, 1) X(3, 11, 3) X(4, 11, 2) X(5, 11, 1)
 
-hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevInst *insts, int n_inst, int max_ntile, int SP,
-                            int layer, hipStream_t stream)
+hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile,
+                            int SP, int layer, hipStream_t stream)
 {
 #define X(id, ts, r)                                                                                  \
     case id:                                                                                          \
-        return marks ? launch_relax_t<ts, r, true>(insts, n_inst, max_ntile, SP, layer, stream)       \
-                     : launch_relax_t<ts, r, false>(insts, n_inst, max_ntile, SP, layer, stream);
+        return marks ? launch_relax_t<ts, r, true>(lay, max_L, n_inst, max_ntile, SP, layer, stream)  \
+                     : launch_relax_t<ts, r, false>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
@@ -656,16 +656,16 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevInst *insts, in
 #undef X
 }
 
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpDevInst *insts, const GdpSched *sched,
-                                  int grid_blocks, int layer0, int layers, hipStream_t stream)
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
+                                  int layers, hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
 #define X(id, ts, r)                                                                                              \
     case id:                                                                                                      \
         if (marks)                                                                                                \
-            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, true>), grid, block, 0, stream, insts, sched, layer0);  \
+            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, true>), grid, block, 0, stream, sched, layer0);  \
         else                                                                                                      \
-            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, false>), grid, block, 0, stream, insts, sched, layer0); \
+            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, false>), grid, block, 0, stream, sched, layer0); \
         break;
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
