@@ -43,8 +43,8 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the relaxation kernel measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (scaled by a copy kernel of known size); see profiles/.  None until measured.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "cfg2": 144.4e6,    # profiles/gdp_relax_kernel_cfg2.txt        (algorithmic 142.6e6)
-    "cfg3": 227.5e9,    # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 188.2e9; one launch per solve)
+    "cfg2": 10.916e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
+    "cfg3": 45.2e9,     # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
 }
 
 
