@@ -58,14 +58,15 @@ struct Group {  // instances with the same S, sorted by L descending
     size_t off_sched, off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
-// Target-tile width: the one that pads S the least (ties: the first).
+// Target-tile width: the one that pads S the least; of two that pad alike the wider one, which
+// issues fewer cost-row loads per relaxation (S = 88: eight blocks of 11 rather than eleven of 8).
 int pick_ts(int S)
 {
     int best = GDP_VARIANTS[0].ts;
     size_t best_sp = align_up((size_t)S, (size_t)best);
     for (int v = 1; v < GDP_NUM_VARIANTS; ++v) {
         const size_t sp = align_up((size_t)S, (size_t)GDP_VARIANTS[v].ts);
-        if (sp < best_sp) { best = GDP_VARIANTS[v].ts; best_sp = sp; }
+        if (sp < best_sp || (sp == best_sp && GDP_VARIANTS[v].ts > best)) { best = GDP_VARIANTS[v].ts; best_sp = sp; }
     }
     return best;
 }
