@@ -1,7 +1,8 @@
 // Host side of libgalvatron_dp_hip.so: the C ABI declared in include/galvatron_dp_hip.h.
 //
-// A plan owns one device allocation, one stream and the events used for timing; nothing is shared
-// between plans, so calls from different threads never touch common mutable state.
+// A plan owns one device allocation, one stream and the events used for timing while it lives, so
+// calls from different threads never touch common mutable state -- but for the cache of device
+// allocations below, which is behind a mutex.
 #include "../../include/galvatron_dp_hip.h"
 #include "gdp_kernels.h"
 
@@ -10,6 +11,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -38,6 +40,101 @@ int fail_hip(hipError_t e, const char *what)
     } while (0)
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---- cache of device allocations -----------------------------------------------------------------
+// Getting fresh device memory costs far more than filling it (94 GB for 256 Llama-7B-like instances:
+// 2.7 s to allocate, 0.05 s to solve), and the search engine solves thousands of DPs in a row.  The
+// allocation of a finished plan is therefore kept for the next plan on that device instead of being
+// freed: up to GALVATRON_DP_CACHE_MB (default 16384, 0 = keep nothing) in total, the largest kept
+// ones given up first when that is exceeded, all of them on an out-of-memory error or gdp_cache_trim().
+struct Arena {
+    int device;
+    char *ptr;
+    size_t bytes;
+};
+std::mutex g_arena_mu;
+std::vector<Arena> g_arenas;
+
+size_t env_mb(const char *name, size_t dflt_mb)
+{
+    const char *e = getenv(name);
+    if (!e || !*e) return dflt_mb << 20;
+    const long long v = atoll(e);
+    return v <= 0 ? 0 : (size_t)v << 20;
+}
+
+void arena_trim(int device /* -1: every device */)
+{
+    std::vector<Arena> drop;
+    {
+        std::lock_guard<std::mutex> lk(g_arena_mu);
+        for (size_t i = 0; i < g_arenas.size();) {
+            if (device < 0 || g_arenas[i].device == device) {
+                drop.push_back(g_arenas[i]);
+                g_arenas.erase(g_arenas.begin() + (long)i);
+            } else {
+                ++i;
+            }
+        }
+    }
+    int cur = 0;
+    (void)hipGetDevice(&cur);
+    for (const Arena &a : drop) {
+        (void)hipSetDevice(a.device);
+        (void)hipFree(a.ptr);
+    }
+    (void)hipSetDevice(cur);
+}
+
+// The smallest kept allocation of `device` that holds `need` bytes, or a fresh one.
+hipError_t arena_take(int device, size_t need, char **ptr, size_t *bytes)
+{
+    {
+        std::lock_guard<std::mutex> lk(g_arena_mu);
+        size_t best = g_arenas.size();
+        for (size_t i = 0; i < g_arenas.size(); ++i)
+            if (g_arenas[i].device == device && g_arenas[i].bytes >= need &&
+                (best == g_arenas.size() || g_arenas[i].bytes < g_arenas[best].bytes))
+                best = i;
+        if (best != g_arenas.size()) {
+            *ptr = g_arenas[best].ptr;
+            *bytes = g_arenas[best].bytes;
+            g_arenas.erase(g_arenas.begin() + (long)best);
+            return hipSuccess;
+        }
+    }
+    hipError_t e = hipMalloc((void **)ptr, need);
+    if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
+        (void)hipGetLastError();
+        arena_trim(device);  // what is kept may be what is missing
+        e = hipMalloc((void **)ptr, need);
+    }
+    *bytes = need;
+    return e;
+}
+
+void arena_give(int device, char *ptr, size_t bytes)
+{
+    const size_t cap = env_mb("GALVATRON_DP_CACHE_MB", 16384);
+    std::vector<Arena> drop;
+    if (bytes > cap) {
+        drop.push_back({device, ptr, bytes});
+    } else {
+        std::lock_guard<std::mutex> lk(g_arena_mu);
+        g_arenas.push_back({device, ptr, bytes});
+        size_t total = 0;
+        for (const Arena &a : g_arenas) total += a.bytes;
+        while (total > cap) {  // the largest first: small ones serve the many small solves
+            size_t big = 0;
+            for (size_t i = 1; i < g_arenas.size(); ++i)
+                if (g_arenas[i].bytes > g_arenas[big].bytes) big = i;
+            total -= g_arenas[big].bytes;
+            drop.push_back(g_arenas[big]);
+            g_arenas.erase(g_arenas.begin() + (long)big);
+        }
+    }
+    for (const Arena &a : drop) (void)hipFree(a.ptr);  // same device as the caller's plan
+}
 
 struct HostInst {
     int orig;  // index in the caller's arrays
@@ -86,7 +183,8 @@ struct gdp_plan {
     std::vector<HostInst> inst;  // sorted order
     std::vector<Group> groups;
     char *dbase = nullptr;
-    size_t dbytes = 0;
+    size_t dbytes = 0;       // bytes laid out
+    size_t dalloc = 0;       // bytes of the allocation behind dbase (a kept one may be larger)
     size_t off_insts = 0, off_keys = 0, off_out = 0, off_res = 0;
     int n_key_total = 0;
     size_t n_res_total = 0;
@@ -126,6 +224,8 @@ int validate(const gdp_problem *p, int i)
     if (!p) return bad(GDP_E_BADARG, "null problem");
     if (p->L < 1 || p->V < 1 || p->S < 1) return bad(GDP_E_BADARG, "L, V and S must be >= 1");
     if (p->S > GDP_MAX_S) return bad(GDP_E_BADARG, "S exceeds GDP_MAX_S");
+    if (p->S > GDP_MAX_S_MARKS && (p->flags & (GDP_KEEP_MARKS | GDP_EXPORT_MARK)))
+        return bad(GDP_E_BADARG, "S exceeds GDP_MAX_S_MARKS and the argmin table was asked for");
     if (!p->mem || !p->intra || !p->inter) return bad(GDP_E_BADARG, "null input array");
     if (p->n_key < 0 || (p->n_key > 0 && (!p->other_mem || !p->other_time)))
         return bad(GDP_E_BADARG, "bad key arrays");
@@ -176,7 +276,11 @@ int validate(const gdp_problem *p, int i)
 void destroy(gdp_plan *pl)
 {
     if (!pl) return;
-    if (pl->dbase) (void)hipFree(pl->dbase);
+    if (pl->dbase) {
+        (void)hipSetDevice(pl->device);
+        if (pl->stream) (void)hipStreamSynchronize(pl->stream);
+        arena_give(pl->device, pl->dbase, pl->dalloc);
+    }
     for (hipEvent_t e : pl->ev_relax) (void)hipEventDestroy(e);
     if (pl->ev_begin) (void)hipEventDestroy(pl->ev_begin);
     if (pl->ev_end) (void)hipEventDestroy(pl->ev_end);
@@ -228,6 +332,16 @@ void fill_bands(const gdp_problem *q, const HostInst &h, int tile_rows, bool ski
         }
         reach = std::min<int64_t>(reach + minfin[(size_t)l], h.V);
     }
+}
+
+// Device bytes one instance takes in the costs-only layout, to within the padding of the rows.
+size_t footprint(const gdp_problem *q)
+{
+    int maxm = 1;
+    for (size_t k = 0; k < (size_t)q->L * q->S; ++k)
+        if (q->mem[k] < q->V) maxm = std::max(maxm, q->mem[k]);
+    const size_t ld = (size_t)q->V + (size_t)maxm + 1024;
+    return sizeof(double) * ((size_t)q->L + 1) * ((size_t)q->S + 1) * ld;
 }
 
 int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
@@ -398,6 +512,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     // One cost buffer per layer lets all layers share a launch and lets the backtrack recompute the
     // argmin of the cells it visits, so that the relaxation does not have to track it.  If that does
     // not fit in device memory: two cost buffers, the argmin table, one launch per layer.
+    int max_S = 0;
+    for (const auto &h : inst) max_S = std::max(max_S, h.S);
+    if (pl->keep_marks && max_S > GDP_MAX_S_MARKS)  // preset from the environment
+        return fail(GDP_E_BADARG, "S exceeds GDP_MAX_S_MARKS and the argmin table is to be kept");
     for (int attempt = 0; attempt < 2; ++attempt) {
         off = fixed_bytes;
         pl->can_fuse = pl->fused || !pl->keep_marks;
@@ -409,11 +527,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
             h.off_M = pl->keep_marks ? take((size_t)h.L * h.S * (size_t)h.ldm) : 0;
         }
         pl->dbytes = off;
-        hipError_t e = hipMalloc((void **)&pl->dbase, pl->dbytes);
+        hipError_t e = arena_take(pl->device, pl->dbytes, &pl->dbase, &pl->dalloc);
         if (e == hipSuccess) break;
         pl->dbase = nullptr;
         (void)hipGetLastError();
-        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse) {
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && max_S <= GDP_MAX_S_MARKS) {
             pl->fused = false;
             pl->keep_marks = true;
             continue;
@@ -779,16 +897,41 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
 
 void gdp_plan_destroy(gdp_plan *plan) { destroy(plan); }
 
+void gdp_cache_trim(void) { arena_trim(-1); }
+
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
 {
+    g_err.clear();
     if (!r) return fail(GDP_E_BADARG, "null results");
-    gdp_plan *pl = nullptr;
-    int rc = gdp_plan_create(n, p, &pl);
-    if (rc != GDP_OK) return rc;
-    rc = run(pl, 0, nullptr);
-    if (rc == GDP_OK) rc = fetch(pl, r);
-    destroy(pl);
-    return rc;
+    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
+    for (int i = 0; i < n; ++i) {  // all of them first: nothing is written when one is rejected
+        int rc = validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+    }
+    // A batch whose cost buffers would take more than GALVATRON_DP_ARENA_MB (default 8192) of device
+    // memory is solved in consecutive parts that reuse one allocation: the time to obtain device
+    // memory grows with its size, the time to solve a part does not grow faster than its share.
+    const size_t budget = std::max<size_t>(env_mb("GALVATRON_DP_ARENA_MB", 8192), (size_t)1 << 20);
+    int begin = 0;
+    while (begin < n) {
+        int end = begin;
+        size_t bytes = 0;
+        while (end < n && end - begin < 65535) {
+            const size_t b = footprint(p[end]);
+            if (end > begin && bytes + b > budget) break;
+            bytes += b;
+            ++end;
+        }
+        gdp_plan *pl = nullptr;
+        int rc = gdp_plan_create(end - begin, p + begin, &pl);
+        if (rc != GDP_OK) return rc;
+        rc = run(pl, 0, nullptr);
+        if (rc == GDP_OK) rc = fetch(pl, r + begin);
+        destroy(pl);
+        if (rc != GDP_OK) return rc;
+        begin = end;
+    }
+    return GDP_OK;
 }
 
 int gdp_solve(const gdp_problem *p, gdp_result *r)

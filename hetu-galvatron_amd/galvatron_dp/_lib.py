@@ -27,14 +27,16 @@ GDP_LAUNCH_FUSED = 4
 GDP_LAUNCH_PER_LAYER = 8
 GDP_COMPUTE_ALL = 16
 GDP_KEEP_MARKS = 32
-GDP_MAX_S = 256
+GDP_MAX_S = 1024
+GDP_MAX_S_MARKS = 256
 GDP_OPT_FUSED = 1
 GDP_OPT_SPIN_LIMIT = 2
 GDP_OPT_POISON = 3
 GDP_OPT_NO_FALLBACK = 4
 
 EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
-                    "gdp_plan_destroy", "gdp_plan_set_option", "gdp_last_error", "gdp_version", "gdp_device_info")
+                    "gdp_plan_destroy", "gdp_plan_set_option", "gdp_cache_trim", "gdp_last_error", "gdp_version",
+                    "gdp_device_info")
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -88,6 +90,8 @@ def lib() -> ctypes.CDLL:
         L.gdp_plan_set_option.restype = ctypes.c_int
         L.gdp_plan_destroy.argtypes = [ctypes.c_void_p]
         L.gdp_plan_destroy.restype = None
+        L.gdp_cache_trim.argtypes = []
+        L.gdp_cache_trim.restype = None
         L.gdp_last_error.argtypes = []
         L.gdp_last_error.restype = ctypes.c_char_p
         L.gdp_version.argtypes = []
@@ -183,6 +187,11 @@ def _arrays(problems: Sequence[Problem]):
     P = (ctypes.POINTER(gdp_problem) * n)(*[ctypes.pointer(p._c_problem) for p in problems])
     R = (ctypes.POINTER(gdp_result) * n)(*[ctypes.pointer(p._c_result) for p in problems])
     return P, R
+
+
+def cache_trim() -> None:
+    """gdp_cache_trim: frees the device allocations that finished plans left behind for reuse."""
+    lib().gdp_cache_trim()
 
 
 def solve_batch(problems: Sequence[Problem]) -> None:

@@ -34,13 +34,14 @@ extern "C" {
 
 /* return codes */
 #define GDP_OK 0
-#define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S above GDP_MAX_S, ... */
+#define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S above GDP_MAX_S(_MARKS), ... */
 #define GDP_E_UNSUPPORTED (-2) /* an input the device recurrence does not cover: mem <= 0 */
 #define GDP_E_NONFINITE (-3)   /* NaN or -inf in a cost array (the reference's result is then order-dependent) */
 #define GDP_E_NOMEM (-4)       /* device or host allocation failed */
 #define GDP_E_HIP (-5)         /* any other HIP runtime error; text in gdp_last_error() */
 
-#define GDP_MAX_S 256 /* strategies per layer (argmin table entries are one byte) */
+#define GDP_MAX_S 1024      /* strategies per layer */
+#define GDP_MAX_S_MARKS 256 /* ... when the argmin table is kept (GDP_KEEP_MARKS, GDP_EXPORT_MARK): its entries are bytes */
 
 /* gdp_problem.flags */
 #define GDP_EXPORT_F 1u    /* write result.f_out    (final f, reference layout [V][S])       */
@@ -53,7 +54,8 @@ extern "C" {
                                    cost buffers of all layers stay in device memory, and the backtrack recomputes
                                    the argmin of the L cells on its path -- same results, two fifths fewer
                                    instructions.  Implied by GDP_EXPORT_MARK; chosen by the library when the
-                                   per-layer cost buffers do not fit in device memory. */
+                                   per-layer cost buffers do not fit in device memory (GDP_E_NOMEM instead if S
+                                   is above GDP_MAX_S_MARKS). */
 
 /* One DP instance == one reference call.  Field <- reference argument (csrc/dp_core.cpp:24-35):
  *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),
@@ -106,7 +108,9 @@ int gdp_solve(const gdp_problem *p, gdp_result *r);
 
 /* Solve n independent instances (e.g. every pipeline stage of every pp_deg, or a whole
  * bsz x chunk sweep: the DPAlg.fit calls issued from dynamic_programming.py:446-488 and
- * search_engine.py:477-498) with one launch grid per layer index. */
+ * search_engine.py:477-498) with one launch grid per layer index.  A batch whose cost buffers would
+ * exceed GALVATRON_DP_ARENA_MB (default 8192) of device memory is solved in consecutive parts that
+ * reuse one allocation. */
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r);
 
 /* The same in three steps, so that a caller (or a benchmark) can keep inputs resident in
@@ -135,6 +139,11 @@ void gdp_plan_destroy(gdp_plan *plan);
 #define GDP_OPT_POISON 3 /* test aid: NaN-fill every not-yet-written cost buffer before each run */
 #define GDP_OPT_NO_FALLBACK 4 /* test aid: an abandoned fused launch is an error, not a switch to per-layer */
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
+
+/* Frees the device allocations that finished plans left behind for reuse (no counterpart in the
+ * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 16384, 0 keeps
+ * nothing), because obtaining device memory costs far more than a solve. */
+void gdp_cache_trim(void);
 
 /* Text of the calling thread's last error ("" if none). */
 const char *gdp_last_error(void);

@@ -60,6 +60,11 @@ def test_validation_happens_before_any_device_work():
     p = _lib.Problem(big_s, np.ones((1, _lib.GDP_MAX_S + 1)), np.zeros((1, _lib.GDP_MAX_S + 1, _lib.GDP_MAX_S + 1)),
                      10, [0], [0.0])
     assert rc_of(p)[0] == _lib.GDP_E_BADARG
+    n = _lib.GDP_MAX_S_MARKS + 1      # the argmin table has byte entries: no table above 256 strategies
+    p = _lib.Problem(np.ones((1, n), np.int32), np.ones((1, n)), np.zeros((1, n, n)), 10, [0], [0.0], export_mark=True)
+    assert rc_of(p)[0] == _lib.GDP_E_BADARG
+    p = _lib.Problem(np.ones((1, n), np.int32), np.ones((1, n)), np.zeros((1, n, n)), 10, [0], [0.0], keep_marks=True)
+    assert rc_of(p)[0] == _lib.GDP_E_BADARG
     assert lib.gdp_plan_create(0, None, ctypes.byref(ctypes.c_void_p())) == _lib.GDP_E_BADARG
 
 

@@ -110,6 +110,31 @@ def test_costs_only_and_mark_table_modes_agree(golden, name, launch, keep_marks)
         assert t.relax_bytes == cells * (17 if keep_marks else 16)
 
 
+def test_batch_solved_in_parts_and_allocation_reuse(golden, monkeypatch):
+    """A batch above the device-memory budget of one allocation is solved in consecutive parts; the
+    allocation of a finished plan is reused by the next one (stale contents must not matter) and
+    can be given back."""
+    names = ["cfg3_smallV_%d" % i for i in range(8)] + ["ties_2", "cfg2_small", "infeasible_4"]
+    insts = [H.build_case(golden[n]) for n in names]
+    monkeypatch.setenv("GALVATRON_DP_ARENA_MB", "1")        # every instance becomes a part of its own
+    for rep in range(2):
+        probs = [_problem(i) for i in insts]
+        _lib.solve_batch(probs)
+        for n, prob in zip(names, probs):
+            _check_against_golden(prob, golden[n], f"{n} rep {rep}")
+    monkeypatch.setenv("GALVATRON_DP_CACHE_MB", "0")        # nothing is kept from here on
+    probs = [_problem(i) for i in insts]
+    _lib.solve_batch(probs)
+    for n, prob in zip(names, probs):
+        _check_against_golden(prob, golden[n], n)
+    _lib.cache_trim()
+    monkeypatch.delenv("GALVATRON_DP_ARENA_MB")
+    probs = [_problem(i) for i in insts]
+    _lib.solve_batch(probs)
+    for n, prob in zip(names, probs):
+        _check_against_golden(prob, golden[n], n)
+
+
 def test_abandoned_fused_launch_falls_back_or_reports(golden):
     """A spin limit of 1 makes waiting wavefronts give up at once (forced from the host; every
     kernel still runs to completion).  With the fallback the plan switches to per-layer launches

@@ -1,8 +1,10 @@
 """Differential test on the GPU: seeded random instances through the plugin signature against
 the C oracle, on shapes chosen to hit the kernel's corners: S around the register-tile widths
-(8, 11) and the wavefront width (63..65, 127..129, 255, 256), V not a multiple of any tile height,
+(8, 11) and the wavefront width (63..65, 127..129, 255..257, 300, 513), V not a multiple of any tile height,
 memory costs near 1, near V and above V, +inf costs, exact ties, shared and per-layer inter
 matrices, start rows below 0.  Full f and mark arrays are compared as well as the results."""
+import os
+
 import numpy as np
 import pytest
 
@@ -15,7 +17,8 @@ pytestmark = pytest.mark.gpu
 SHAPES = [(1, 1, 1), (1, 1, 7), (2, 1, 64), (3, 2, 65), (4, 7, 191), (3, 8, 192), (5, 9, 193), (2, 10, 255),
           (6, 11, 256), (3, 12, 257), (4, 16, 383), (2, 21, 385), (7, 22, 512), (3, 23, 700), (2, 33, 129),
           (3, 44, 1000), (2, 45, 130), (2, 63, 300), (3, 64, 333), (2, 65, 200), (2, 88, 410), (1, 127, 150),
-          (2, 128, 140), (2, 129, 131), (1, 255, 90), (2, 256, 70), (9, 5, 2048), (12, 3, 4099), (20, 4, 1500)]
+          (2, 128, 140), (2, 129, 131), (1, 255, 90), (2, 256, 70), (9, 5, 2048), (12, 3, 4099), (20, 4, 1500),
+          (2, 257, 70), (2, 300, 150), (1, 513, 40)]
 
 
 def _compare(inst, tag, launch=None):
@@ -25,7 +28,7 @@ def _compare(inst, tag, launch=None):
     keys = sorted(inst.other_mem)
     wt, wr, wm, wf, wmark = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time,
                                     keep=True)
-    for marks in (False, True):
+    for marks in ((False, True) if inst.S <= _lib.GDP_MAX_S_MARKS else (False,)):   # mark entries are bytes
         prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
                             [inst.other_time[k] for k in keys], inter_index=inst.inter_index, export_f=True,
                             export_mark=marks, launch=launch)
@@ -45,6 +48,8 @@ def _compare(inst, tag, launch=None):
 @pytest.mark.parametrize("n,shape", list(enumerate(SHAPES)))
 def test_random_instances_against_oracle(n, shape):
     L, S, V = shape
+    if S > _lib.GDP_MAX_S_MARKS and os.environ.get("GALVATRON_DP_KEEP_MARKS", "0") != "0":
+        pytest.skip("the environment forces the argmin table, whose entries are bytes")
     for variant in range(4):
         rng = np.random.Generator(np.random.PCG64([77, n, variant]))
         ties = variant in (1, 3)
