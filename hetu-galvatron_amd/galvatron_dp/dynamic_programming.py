@@ -9,16 +9,17 @@ calls the plugin once per stage; here every stage of every pipeline degree that 
 (``galvatron_dp_core.dynamic_programming_core_batch``), and the O(S^2) pairwise inter-layer cost
 table is built once per (pp_deg, layer type) from per-strategy feature vectors.
 
-The cost models stay the caller's: ``memcost_model`` / ``timecost_model`` are passed in exactly as
-the reference passes them (dynamic_programming.py:129-150); ``OtherTimeCostModel`` and
-``pipeline_costmodel`` (imported by the reference from its own cost_model.py, :3-4) are taken from
-the ``other_timecost_model`` / ``pipeline_costmodel`` keyword arguments.
+``memcost_model`` / ``timecost_model`` are passed in exactly as the reference passes them
+(dynamic_programming.py:129-150); ``OtherTimeCostModel`` and ``pipeline_costmodel`` (which the
+reference imports from its own cost_model.py, :3-4) are taken from the ``other_timecost_model`` /
+``pipeline_costmodel`` keyword arguments and default to ``galvatron_dp.cost_models``.
 """
 from __future__ import annotations
 
 import numpy as np
 
 import galvatron_dp_core
+from . import cost_models
 
 __all__ = ["DPAlg", "DpOnModel"]
 
@@ -135,7 +136,7 @@ class _Prepared:
 
 class DpOnModel:
     """Same constructor arguments as the reference (dynamic_programming.py:129-150) plus the two
-    callables the reference imports from its cost_model.py."""
+    callables the reference imports from its cost_model.py (default: this package's)."""
 
     def __init__(self, strategies_set, memcost_model, timecost_model, model_args_list=None, train_args_list=None,
                  parallel_args_list=None, profile_model_args_list=None, profile_hardware_args_list=None,
@@ -146,8 +147,8 @@ class DpOnModel:
         self.strategies_set = strategies_set
         self.memcost_model = memcost_model
         self.timecost_model = timecost_model
-        self.other_timecost_model = other_timecost_model
-        self.pipeline_costmodel = pipeline_costmodel
+        self.other_timecost_model = other_timecost_model or cost_models.OtherTimeCostModel
+        self.pipeline_costmodel = pipeline_costmodel or cost_models.pipeline_costmodel
         self.model_args_list = model_args_list
         self.train_args_list = train_args_list
         self.parallel_args_list = parallel_args_list

@@ -160,6 +160,56 @@ def build(DpOnModel, cfg, **extra):
                      **extra)
 
 
+# ---- scenarios with the real cost models ------------------------------------------------------------
+# The whole producer -> DP -> pipeline-model chain: the reference's DpOnModel fed by the reference's
+# MemoryCostModel / TimeCostModel / OtherTimeCostModel / pipeline_costmodel on one side, this
+# repository's classes on the other, over a synthetic profile (tests/cost_model_cases.py).
+REAL_SCENARIOS = ['real_flush', 'real_gpipe_two_types', 'real_tight_zero2', 'real_vsp_embed_sdp']
+
+
+def real_scenario(name):
+    base = dict(layer_num=[12], pipeline_type='pipedream_flush', micro=True, sp=True, fine=1, max_mem=24000,
+                bsz=64, min_tp=1, max_tp=8, vsp=0, embed_sdp=0, sp_search=1, mbsz={1: 8, 2: 4, 4: 2},
+                pps=(1, 2, 4), stage={1: [12], 2: [7, 5], 4: [4, 3, 3, 2]}, seq=[2048], profile_seeds=[11],
+                params=[120.0], zero2=False, sp_space='tp+sp', mixed=True)
+    table = {
+        'real_flush': {},
+        'real_gpipe_two_types': {'layer_num': [6, 6], 'pipeline_type': 'gpipe', 'seq': [2048, 512],
+                                 'profile_seeds': [5, 6], 'params': [150.0, 60.0], 'sp_space': 'tp', 'max_mem': 30000},
+        'real_tight_zero2': {'max_mem': 9000, 'zero2': True, 'params': [220.0], 'profile_seeds': [23], 'mixed': False},
+        'real_vsp_embed_sdp': {'vsp': 1, 'embed_sdp': 1, 'profile_seeds': [31], 'bsz': 32, 'max_mem': 16000},
+    }
+    cfg = dict(base)
+    cfg.update(table[name])
+    return cfg
+
+
+def build_real(DpOnModel, cost_mod, args_mod, cfg, **extra):
+    """DpOnModel over ``cost_mod``'s MemoryCostModel / TimeCostModel and ``args_mod``'s argument
+    records (the reference's modules or galvatron_dp.cost_models for both)."""
+    import cost_model_cases as C
+    n = len(cfg['layer_num'])
+    lists = [[], [], [], [], []]
+    for i in range(n):
+        prof = C.profile(np.random.Generator(np.random.PCG64([99, cfg['profile_seeds'][i]])))
+        model = dict(parameter_size=cfg['params'][i], seq_length=cfg['seq'][i], hidden_size=4096, layer_num=24)
+        train = dict(mixed_precision=cfg['mixed'], async_grad_reduce=True, pytorch_context_mem=1024)
+        parallel = dict(use_zero2_for_dp=cfg['zero2'], disable_vtp=False, sequence_parallel=cfg['sp'],
+                        sp_space=cfg['sp_space'], pipeline_type=cfg['pipeline_type'],
+                        optimal_chunk_func=C.chunk_func, chunks=None)
+        for lst, rec in zip(lists, C._records(args_mod, prof, model, train, parallel)):
+            lst.append(rec)
+    config = SimpleNamespace(hidden_size=4096, mixed_precision='bf16' if cfg['mixed'] else 'fp32',
+                             sequence_parallel=cfg['sp'], global_memory_buffer=True, fine_grained_mode=cfg['fine'])
+    return DpOnModel(strategies(8, cfg['pps']), cost_mod.MemoryCostModel, cost_mod.TimeCostModel,
+                     model_args_list=lists[0], train_args_list=lists[1], parallel_args_list=lists[2],
+                     profile_model_args_list=lists[3], profile_hardware_args_list=lists[4], max_mem=cfg['max_mem'],
+                     layer_num=list(cfg['layer_num']), sequence_len=list(cfg['seq']), multi_layer_type=True,
+                     pp_stage_dict={k: list(v) for k, v in cfg['stage'].items()},
+                     comm_coe_dict=lists[4][0].comm_coe_dict, gpu_num=8, model_microbatch_after_dp=cfg['micro'],
+                     pipeline_type=cfg['pipeline_type'], config=config, **extra)
+
+
 def run(dpm, cfg):
     fit = dpm.fit(cfg['bsz'], cfg['min_tp'], cfg['max_tp'], cfg['vsp'], cfg['embed_sdp'], cfg['sp_search'],
                   print_=False, mbsz_dict=dict(cfg['mbsz']))

@@ -1,0 +1,140 @@
+"""The cost models (galvatron_dp/cost_models.py) against numbers recorded from the reference's
+classes (tests/golden/cost_model_golden.json, written by tests/golden/make_cost_model_golden.py)
+on seeded scenarios, bit for bit (floats as hex), plus closed forms that pin single terms
+independently of the fixture."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import cost_model_cases as C
+from galvatron_dp import cost_models as M
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def golden():
+    with open(os.path.join(HERE, "golden", "cost_model_golden.json")) as fh:
+        return json.load(fh)
+
+
+@pytest.mark.parametrize("kind,runner", [("memory", C.run_memory), ("time", C.run_time), ("other", C.run_other),
+                                         ("pipeline", C.run_pipeline)])
+def test_bit_identical_to_recorded_reference_outputs(golden, kind, runner):
+    assert len(golden[kind]) >= 100
+    for rec in golden[kind]:
+        got = runner(M, M, rec["case"])
+        assert got == rec["want"], f"{kind} case {rec['case']}"
+
+
+def test_strategy_text_round_trip(golden):
+    for rec in golden["strings"]:
+        assert M.form_strategy(rec["strategy"]) == rec["text"]
+        assert M.strategy_str2list(rec["text"]) == rec["back"]
+
+
+def test_micro_batch_split_is_torch_chunk():
+    # torch.arange(10).chunk(4) -> sizes 3,3,3,1; .chunk(6) of 9 gives 5 pieces of 2,2,2,2,1
+    assert [len(p) for p in M.chunk_like_torch(10, 4)] == [3, 3, 3, 1]
+    assert [len(p) for p in M.chunk_like_torch(9, 6)] == [2, 2, 2, 2, 1]
+    assert M.get_real_chunk(9, 6) == 5 and M.get_real_chunk(9, 1) == 1
+    with pytest.raises(ValueError):
+        M.chunk_like_torch(4, 0)
+    assert M.get_time_cost_all_stages([1.0, 2.0, 4.0, 8.0], [1, 3]) == [1.0, 14.0]
+
+
+def _args(**over):
+    line = {"popt": [0.02, 0.1]}
+    hw = M.ProfileHardwareArgs(allreduce_dict={2: line, 4: line, 8: line}, all2all_dict={2: line, 4: line, 8: line})
+    return dict(model_args=M.ModelArgs(parameter_size=48, seq_length=512, hidden_size=1024, layer_num=24),
+                train_args=M.TrainArgs(mixed_precision=over.get("mixed", False)),
+                parallel_args=M.ParallelArgs(sp_space="tp"), profile_model_args=M.ProfileModelArgs(),
+                profile_hardware_args=hw)
+
+
+def test_time_model_closed_forms():
+    # pure data parallel, 8 ranks: ring all-reduce volume 2(d-1)/d * parameters per layer
+    t = M.TimeCostModel([1, 1, 8, {"fsdp": 0}], 64, **_args())
+    assert t.dp_message_size == (2 * 7 / 8 * 48) * 24
+    assert t.fct == 35 / 24 * 8 / 1 * 24 and t.bct == t.fct * 2
+    assert t.dc == M.ProfileHardwareArgs().comm_coe_dict["8"]
+    # mixed precision halves it; ZeRO-3 gathers half of the volume once more in the forward pass
+    t16 = M.TimeCostModel([1, 1, 8, {"fsdp": 1}], 64, **_args(mixed=True))
+    assert t16.dp_message_size == t.dp_message_size / 2
+    assert t16.fsdp_allgather_message_size == t16.dp_message_size * 0.5
+    plain = M.TimeCostModel([1, 1, 8, {"fsdp": 0}], 64, **_args(mixed=True))
+    assert t16.gen_result() > plain.gen_result()
+    # no parallelism at all: forward + backward, per layer, in seconds
+    one = M.TimeCostModel([1, 1, 1, {}], 8, **_args())
+    assert one.gen_result() == (one.fct + one.bct) * 0.001 / 24
+    # tensor parallel over consecutive ranks uses the '<tp>_1' coefficient, the other layout '<tp>_0'
+    a = M.TimeCostModel([1, 2, 4, {"tp": 1, "fsdp": 0}], 64, **_args())
+    b = M.TimeCostModel([1, 2, 4, {"tp": 0, "fsdp": 0}], 64, **_args())
+    coe = M.ProfileHardwareArgs().comm_coe_dict
+    assert a.tp_communication_time == a.tp_message_size * coe["2_1"]
+    assert b.tp_communication_time == b.tp_message_size * coe["2_0"]
+    assert a.dc == coe["4_0"] and b.dc == coe["4_1"]
+    # checkpointing: one more forward in the backward pass, half again as many activation collectives
+    c = M.TimeCostModel([1, 2, 4, {"tp": 1, "fsdp": 0, "cpt": 1}], 64, **_args())
+    assert c.bct == a.bct + a.fct and c.tp_message_size == a.tp_message_size * 1.5
+    # the overlap model: whichever of all-reduce and backward is longer keeps running alone afterwards
+    over, rest, flag = a.bct_dp_overlap(a.dp_message_size, a.bct)
+    assert flag is False and over <= a.bct * 1.3 and rest >= 0
+
+
+def test_memory_model_closed_forms():
+    prof = M.ProfileModelArgs(tp_activation_per_bsz_dict={1: 85, 2: 47, 4: 28, 8: 18.5, "checkpoint": 10.0},
+                              other_memory_pp_off={"model_states": {1: 640, 2: 320, 4: 160, 8: 80},
+                                                   "activation": {1: 320, 2: 160, 4: 80, 8: 40}},
+                              other_memory_pp_on={s: {"model_states": {1: 640, 2: 320, 4: 160, 8: 80},
+                                                      "activation": {1: 320, 2: 160, 4: 80, 8: 40}}
+                                                  for s in ("first_stage", "last_stage")})
+    kw = dict(global_batch_size=32, mbsz=4, min_tp=1, max_tp=8, model_args=M.ModelArgs(parameter_size=48),
+              train_args=M.TrainArgs(mixed_precision=True), profile_model_args=prof)
+    par = lambda **o: M.ParallelArgs(optimal_chunk_func=C.chunk_func, **o)          # noqa: E731
+    dp = M.MemoryCostModel([1, 1, 8, {"fsdp": 0}], parallel_args=par(), **kw)
+    assert dp.chunks == 1 and dp.bsz == 4.0 and dp.sdp_size == 8
+    cost = dp.get_memory_cost()
+    assert cost["parameter"] == 48 and cost["model_states"] == 4 * 48 and cost["activation"] == 85 * 4.0
+    assert cost["enc_total"] == cost["model_states"] + cost["activation"]
+    assert sorted(cost["other"]) == [1, 2, 4, 8]
+    assert cost["other"][1] == [640 * 1.0 + 320 * (32 * 1 / 1 / 8 / 1) + 1024]
+    # ZeRO-3 over 8 ranks, one micro-batch: states shrink to 1/8 (+ the 0.003 margin)
+    z3 = M.MemoryCostModel([1, 1, 8, {"fsdp": 1}], parallel_args=par(), **kw)
+    assert z3.get_memory_cost()["model_states"] == 4 * 48 * (1 / 8 + 0.003)
+    # tensor parallel divides the parameters, Ulysses does not and shards over tp*dp instead
+    tp = M.MemoryCostModel([1, 4, 2, {"fsdp": 1, "tp": 1}], parallel_args=par(), **kw)
+    ul = M.MemoryCostModel([1, 4, 2, {"fsdp": 1, "tp": 1, "sp": 1}], parallel_args=par(), **kw)
+    assert tp.parameter_size == 12 and ul.parameter_size == 48 and tp.sdp_size == 2 and ul.sdp_size == 8
+    # checkpointed activations, divided over tp only with sequence parallelism
+    ck = M.MemoryCostModel([1, 2, 4, {"fsdp": 0, "tp": 1, "cpt": 1}], parallel_args=par(sequence_parallel=True), **kw)
+    ck0 = M.MemoryCostModel([1, 2, 4, {"fsdp": 0, "tp": 1, "cpt": 1}], parallel_args=par(), **kw)
+    assert ck.activation_size == 10.0 * ck.bsz / 2 and ck0.activation_size == 10.0 * ck0.bsz
+    # 1F1B: stage 0 of 4 holds min(4, chunks) micro-batches, the last stage one
+    f = [M.MemoryCostModel([4, 1, 2, {"fsdp": 0}], stage_idx=i, parallel_args=par(pipeline_type="pipedream_flush"), **kw)
+         for i in range(4)]
+    assert [m.chunks for m in f] == [4] * 4
+    assert [m.act_1f1b_ratio for m in f] == [1.0, 0.75, 0.5, 0.25]
+    g = M.MemoryCostModel([4, 1, 2, {"fsdp": 0}], parallel_args=par(pipeline_type="gpipe"), **kw)
+    assert g.bsz == 4                                        # one micro-batch of 16/4 samples
+    with pytest.raises(AssertionError):
+        M.MemoryCostModel([1, 1, 8, {}], parallel_args=par(), global_batch_size=8, min_tp=1, model_args=M.ModelArgs(),
+                          train_args=M.TrainArgs(), profile_model_args=prof)       # mbsz missing
+
+
+def test_pipeline_model_degenerate_cases():
+    assert M.pipeline_costmodel(M.TimeCostModel, [4], [], [], [], [], [], None, [2, 2], 4, 32, 1, [0, 0]) == np.inf
+    stage, total = M.pipeline_costmodel(M.TimeCostModel, [4], [], [], [], [], [], None, [2, 2], 4, 32, 1, [0, 0],
+                                        return_stage_cost=True)
+    assert stage == [np.inf, np.inf] and total == np.inf
+    # one stage, one micro-batch, nothing else: the sum of the layers' times
+    a = _args()
+    lists = [[a["model_args"]], [a["train_args"]], [a["parallel_args"]], [a["profile_model_args"]],
+             [a["profile_hardware_args"]]]
+    s = [1, 1, 8, {"fsdp": 0}]
+    total = M.pipeline_costmodel(M.TimeCostModel, [3], *lists, [s, s, s], [3], 1, 64, 1, [0.0])
+    one = M.TimeCostModel(s, 64, **a).gen_result()
+    compute = M.TimeCostModel(s, 64, no_comm=True, **a).gen_result()
+    assert total == np.sum([compute] * 3) + max(np.sum([one] * 3) - np.sum([compute] * 3), 0)

@@ -32,6 +32,18 @@ def test_dp_on_model_matches_reference(want, name):
     assert got == want[name]
 
 
+@pytest.mark.parametrize("name", stubs.REAL_SCENARIOS)
+def test_cost_models_dp_and_pipeline_model_together_match_reference(want, name):
+    """Producer -> DP -> pipeline model: this repository's cost models, DpOnModel and HIP core against
+    the reference's cost models, DpOnModel and compiled dp_core on the same synthetic profile."""
+    from galvatron_dp import cost_models
+    from galvatron_dp.dynamic_programming import DpOnModel
+    cfg = stubs.real_scenario(name)
+    dpm = stubs.build_real(DpOnModel, cost_models, cost_models, cfg)
+    got = stubs.run(dpm, cfg)
+    assert got == want[name]
+
+
 def test_dpalg_fit_matches_plugin_semantics(golden):
     from galvatron_dp.dynamic_programming import DPAlg
     rec = golden["galvatron_like"]
