@@ -8,11 +8,11 @@ coefficients keyed '<size>' or '<size>_<0|1>', fitted lines ('popt') for sequenc
 collectives."""
 import numpy as np
 
-N_MEMORY, N_TIME, N_OTHER, N_PIPELINE = 400, 400, 200, 120
+N_MEMORY, N_TIME, N_OTHER, N_PIPELINE, N_PP = 400, 400, 200, 120, 150
 
 
 def _rng(kind, seed):
-    return np.random.Generator(np.random.PCG64([{"memory": 1, "time": 2, "other": 3, "pipeline": 4}[kind], seed]))
+    return np.random.Generator(np.random.PCG64([{"memory": 1, "time": 2, "other": 3, "pipeline": 4, "pp": 5}[kind], seed]))
 
 
 def hexf(x):
@@ -30,8 +30,8 @@ def jsonable(x):
         return int(x)
     if isinstance(x, (float, np.floating)):
         return hexf(x)
-    if x is None:
-        return None
+    if x is None or isinstance(x, str):
+        return x
     raise TypeError(type(x))
 
 
@@ -283,3 +283,53 @@ def run_pipeline(mod, args_mod, seed):
     only = mod.pipeline_costmodel(mod.TimeCostModel, c['layer_num_list'], *lists, strategies, c['partition'],
                                   c['chunks'], c['bsz'], c['min_tp'], c['other_time_cost'])
     return jsonable({'stage': list(stage), 'total': total, 'only': only})
+
+
+# ---- pipeline division ------------------------------------------------------------------------------
+def pp_case(seed):
+    rng = _rng("pp", seed)
+    n_types = int(rng.integers(1, 3))
+    layer_num = [int(rng.integers(4, 33)) for _ in range(n_types)]
+    pp = int(rng.choice([1, 2, 4, 8]))
+    strategies = [s for s in all_strategies() if rng.random() < 0.6 or s[0] == pp]
+    if rng.random() < 0.1:
+        strategies = [s for s in strategies if s[0] != pp]           # nothing to choose from -> (None, None)
+    rng.shuffle(strategies)
+    profs = [profile(rng) for _ in range(n_types)]
+    records = [_common(rng) for _ in range(n_types)]
+    mbsz = {1: int(rng.choice([4, 8])), 2: int(rng.choice([2, 4])), 4: int(rng.choice([1, 2])), 8: 1}
+    return dict(layer_num=layer_num, pp=pp, strategies=[list(s) for s in strategies], profs=profs, records=records,
+                bsz=int(rng.choice([32, 64, 128])), mbsz=mbsz, even=bool(rng.integers(0, 2)))
+
+
+def pp_cases():
+    return list(range(N_PP))
+
+
+def run_pp(pp_mod, args_mod, seed):
+    """``pp_mod`` holds the division functions (the reference's search_engine module or
+    galvatron_dp.pp_utils)."""
+    c = pp_case(seed)
+    lists = [[], [], [], [], []]
+    for prof, (model, train, parallel) in zip(c['profs'], c['records']):
+        for lst, rec in zip(lists, _records(args_mod, prof, model, train, parallel)):
+            lst.append(rec)
+    m, t, p, pm, _ = lists
+    division, per_stage = pp_mod.pp_division_memory_balanced(m, t, p, pm, c['layer_num'], c['pp'], c['bsz'],
+                                                             c['mbsz'][c['pp']], c['strategies'])
+    out = {'division': None if division is None else [int(x) for x in division],
+           'per_stage': None if per_stage is None else list(per_stage),
+           'types_untouched': [x.pipeline_type for x in p]}
+    if any(s[0] == c['pp'] for s in c['strategies']):
+        stage = pp_mod.get_pp_stage_for_bsz([s for s in c['strategies'] if s[0] <= 4], m, t, p, pm, c['layer_num'],
+                                            c['bsz'], c['mbsz'], single_layer_even=c['even'])
+        out['stage_dict'] = {k: None if v is None else [int(x) for x in v] for k, v in stage.items()}
+        world = 8
+        out['chunks'] = pp_mod.check_optimal_chunks(world, [s for s in c['strategies'] if s[0] <= 4],
+                                                    pp_mod.optimal_chunk_func_default, c['bsz'], c['mbsz'], 1)
+    costs = [float(i) * 1.5 + 0.25 for i in range(sum(c['layer_num']) + seed % 3)]
+    even = pp_mod.pp_division_even(c['layer_num'], c['pp'])
+    out['even'] = [int(x) for x in even]
+    out['stage_sums'] = pp_mod.get_cost_all_stages(costs, even if c['pp'] > 1 or seed % 3 < 2 else [sum(c['layer_num'])])
+    out['layer_costs'] = pp_mod.get_layer_costs(c['layer_num'], [1.5, 2.5][:len(c['layer_num'])])
+    return jsonable(out)

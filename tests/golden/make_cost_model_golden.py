@@ -1,6 +1,7 @@
 """Writes tests/golden/cost_model_golden.json: what the REFERENCE's cost models
 (galvatron/core/search_engine/cost_model.py: MemoryCostModel :10-219, TimeCostModel :221-466,
-OtherTimeCostModel :468-658, pipeline_costmodel :695-767) return for seeded random scenarios over
+OtherTimeCostModel :468-658, pipeline_costmodel :695-767) and its pipeline-division utilities
+(search_engine.py:972-1104) return for seeded random scenarios over
 synthetic profiles of the shape the reference's mock profiles have (tests/utils/search_configs.py:
 per-tp activation tables, model-state tables per vocabulary tp degree, collective coefficients keyed
 '<size>' / '<size>_<0|1>', fitted lines for the sequence-parallel collectives).  Run in the build
@@ -39,9 +40,16 @@ def reference_module():
     spec.loader.exec_module(su)
     g = types.ModuleType("galvatron")
     g.__path__ = []
+    # galvatron.utils without its __init__ (which pulls torch-based training helpers): the two plain
+    # modules the search engine needs, their public names gathered on the stand-in package
     gu = types.ModuleType("galvatron.utils")
-    gu.form_strategy, gu.strategy_str2list = su.form_strategy, su.strategy_str2list
+    gu.__path__ = ["/root/reference/galvatron/utils"]
     sys.modules["galvatron"], sys.modules["galvatron.utils"] = g, gu
+    for name in ("strategy_utils", "config_utils"):
+        sub = importlib.import_module("galvatron.utils." + name)
+        for k, v in vars(sub).items():
+            if not k.startswith("_"):
+                setattr(gu, k, v)
     mod = importlib.import_module("_ref_search_engine.cost_model")
     args = importlib.import_module("_ref_search_engine.cost_model_args")
     return mod, args, su
@@ -49,7 +57,10 @@ def reference_module():
 
 def main():
     mod, args, su = reference_module()
-    out = {"memory": [], "time": [], "other": [], "pipeline": [], "strings": []}
+    out = {"memory": [], "time": [], "other": [], "pipeline": [], "strings": [], "pp": []}
+    engine = importlib.import_module("_ref_search_engine.search_engine")      # pipeline-division utilities, :972-1104
+    for case in C.pp_cases():
+        out["pp"].append({"case": case, "want": C.run_pp(engine, args, case)})
     for case in C.memory_cases():
         out["memory"].append({"case": case, "want": C.run_memory(mod, args, case)})
     for case in C.time_cases():

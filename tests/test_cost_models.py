@@ -10,6 +10,7 @@ import pytest
 
 import cost_model_cases as C
 from galvatron_dp import cost_models as M
+from galvatron_dp import pp_utils as PP
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -27,6 +28,29 @@ def test_bit_identical_to_recorded_reference_outputs(golden, kind, runner):
     for rec in golden[kind]:
         got = runner(M, M, rec["case"])
         assert got == rec["want"], f"{kind} case {rec['case']}"
+
+
+def test_pipeline_division_bit_identical_to_recorded_reference_outputs(golden):
+    assert len(golden["pp"]) >= 100
+    kinds = set()
+    for rec in golden["pp"]:
+        got = C.run_pp(PP, M, rec["case"])
+        assert got == rec["want"], f"pp case {rec['case']}"
+        kinds.add("none" if rec["want"]["division"] is None else len(rec["want"]["division"]))
+    assert {"none", 1, 2, 4, 8} <= kinds          # every pipeline degree and the no-candidate case occur
+
+
+def test_pipeline_division_closed_forms():
+    assert PP.pp_division_even([10], 4) == [2, 2, 2, 4] and PP.pp_division_even([6, 6], 1) == [12]
+    assert PP.get_layer_costs([2, 3], [1.0, 5.0]) == [1.0, 1.0, 5.0, 5.0, 5.0]
+    # a leading entry for the non-layer memory goes to the first stage, a trailing one to the last
+    assert PP.get_cost_all_stages([1, 2, 3, 4], [2, 2]) == [3, 7]
+    assert PP.get_cost_all_stages([10, 1, 2, 3, 4], [2, 2]) == [13, 7]
+    assert PP.get_cost_all_stages([10, 1, 2, 3, 4, 20], [2, 2]) == [13, 27]
+    assert PP.optimal_chunk_func_default(16, [2, 2, 2, {}], 3, 1) == 3.0      # ceil((16 // 2) / 3)
+    assert PP.optimal_chunk_func_default(0, [1, 1, 8, {}], 4, 1) == 1
+    assert PP.check_optimal_chunks(8, [[1, 1, 8, {}], [2, 1, 4, {}]], PP.optimal_chunk_func_default, 64,
+                                   {1: 4, 2: 2}, 1) == {1: 2.0, 2: 8.0}
 
 
 def test_strategy_text_round_trip(golden):
