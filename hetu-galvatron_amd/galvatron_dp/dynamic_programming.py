@@ -246,41 +246,46 @@ class DpOnModel:
         big = np.maximum(tp_i, tp_j)
         volume = (big - 1) / big * mbsz * (big // min_tp) * sample_num      # same order of operations
         cost = np.where(redistribute, volume, 0.0)
-        # communication coefficient of the wider of the two tensor-parallel groups
+        # communication coefficient of the wider of the two tensor-parallel groups: the plain one when
+        # that group is everything (or there is no data parallelism beside it), else by the layout
+        # flag of the strategy that owns the wider group
         small_dp = np.minimum(dp[:, None], dp[None, :])
+        plain = (big == 1) | (small_dp == 1)
+        owner_flag = np.where(tp_j > tp_i, tp_flag[None, :], tp_flag[:, None])
+        assert np.isin(owner_flag[~plain], (0, 1)).all()
         coe = np.empty((S, S), dtype=np.float64)
-        for i in range(S):
-            for j in range(S):
-                t = int(big[i, j])
-                if t == 1 or small_dp[i, j] == 1:
-                    key = '%d' % t if '%d' % t in self.comm_coe_dict else '%d_1' % t
-                else:
-                    info = strategy_set[j][-1] if tp[j] > tp[i] else strategy_set[i][-1]
-                    assert 'tp' in info and info['tp'] in [0, 1]
-                    key = '%d_1' % t if info['tp'] else '%d_0' % t
-                coe[i, j] = self.comm_coe_dict[key]
+        table = self.comm_coe_dict
+        for t in np.unique(big):
+            t = int(t)
+            here = big == t
+            if (here & plain).any():
+                coe[here & plain] = table['%d' % t] if '%d' % t in table else table['%d_1' % t]
+            for flag in (0, 1):
+                pick = here & ~plain & (owner_flag == flag)
+                if pick.any():
+                    coe[pick] = table['%d_%d' % (t, flag)]
         cost = cost * coe * 1e-7
-        # tiny ordering biases between strategies that differ only in sp / fsdp / cpt
-        for i in range(S):
-            a = strategy_set[i]
-            for j in range(S):
-                if i == j:
-                    continue
-                b = strategy_set[j]
-                opt = b[-1]
-                if _same_strategy(a, b, ('sp',)) and opt.get('sp'):
-                    cost[i, j] = 1e-10
-                only_fsdp = _same_strategy(a, b, ('fsdp',))
-                only_cpt = _same_strategy(a, b, ('cpt',))
-                if only_fsdp and opt.get('fsdp'):
-                    cost[i, j] = 1e-9
-                if only_cpt and opt.get('cpt'):
-                    cost[i, j] = 2e-9
-                if _same_strategy(a, b, ('fsdp', 'cpt')):
-                    if opt.get('fsdp') and opt.get('cpt'):
-                        cost[i, j] = 3e-9
-                    if not only_fsdp and not only_cpt and a[-1].get('fsdp') and opt.get('cpt'):
-                        cost[i, j] = 1e-9
+        # tiny ordering biases between strategies that differ only in sp / fsdp / cpt.  "Same apart
+        # from key k" (the reference's match_strategy, dynamic_programming.py:196-210) is equality of
+        # (pp, tp, dp) and of the option dictionaries with k removed; the rules are applied in the
+        # reference's order, later ones overriding earlier ones.
+        def same_apart_from(*ignore):
+            ids, seen = [], {}
+            for st in strategy_set:
+                key = (tuple(int(x) for x in st[:3]), frozenset((k, v) for k, v in st[-1].items() if k not in ignore))
+                ids.append(seen.setdefault(key, len(seen)))
+            ids = np.array(ids)
+            return ids[:, None] == ids[None, :]
+
+        on = lambda name: np.array([bool(st[-1].get(name)) for st in strategy_set])       # noqa: E731
+        sp_j, fsdp_j, cpt_j, fsdp_i = on('sp')[None, :], on('fsdp')[None, :], on('cpt')[None, :], on('fsdp')[:, None]
+        off_diagonal = ~np.eye(S, dtype=bool)
+        only_fsdp, only_cpt, both_keys = same_apart_from('fsdp'), same_apart_from('cpt'), same_apart_from('fsdp', 'cpt')
+        cost[off_diagonal & same_apart_from('sp') & sp_j] = 1e-10
+        cost[off_diagonal & only_fsdp & fsdp_j] = 1e-9
+        cost[off_diagonal & only_cpt & cpt_j] = 2e-9
+        cost[off_diagonal & both_keys & fsdp_j & cpt_j] = 3e-9
+        cost[off_diagonal & both_keys & ~only_fsdp & ~only_cpt & fsdp_i & cpt_j] = 1e-9
         return cost
 
     def _inter_cost(self, strategy_set, mbsz, min_tp):
@@ -434,10 +439,10 @@ class DpOnModel:
             else:
                 print(line, flush=True)
 
-    def fit(self, bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, print_=True, mbsz_dict=None):
-        """Same arguments and return value as the reference (dynamic_programming.py:515-565):
-        ``(min_comm_cost, min_res_list, min_pp_deg, min_mem_remain, min_mem_cost, min_vtp)``.
-        All pipeline degrees are prepared first and their DP instances solved in one device batch."""
+    def fit_begin(self, bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, mbsz_dict=None):
+        """First half of ``fit``: prepares every pipeline degree and returns ``(ticket, dps)``.  The
+        caller solves ``dps`` (``DPAlg.fit_many``, alone or together with the instances of other
+        ``fit_begin`` calls: a whole sweep in one device batch) and hands the results to ``fit_end``."""
         if mbsz_dict is None:
             mbsz_dict = {pp_deg: 8 for pp_deg in self.ppdeg_set}
         todo = []
@@ -449,7 +454,13 @@ class DpOnModel:
                 assert self.multi_layer_type
             todo.append((pp_deg, self._prepare(pp_deg, bsz, mbsz_dict[pp_deg], min_tp, max_tp, vsp, embed_sdp,
                                                sp_search) if divisible else None))
-        fits = DPAlg.fit_many([dp for _, P in todo if P is not None for dp in P.dps])
+        ticket = (todo, (bsz, min_tp, max_tp, vsp, embed_sdp, sp_search))
+        return ticket, [dp for _, P in todo if P is not None for dp in P.dps]
+
+    def fit_end(self, ticket, fits, print_=True):
+        """Second half of ``fit``: ``fits`` are the results of the instances ``fit_begin`` returned, in
+        the same order."""
+        todo, (bsz, min_tp, max_tp, vsp, embed_sdp, sp_search) = ticket
         best = (np.inf, None, -1, -1, -1, -1)
         pos = 0
         for pp_deg, P in todo:
@@ -470,3 +481,10 @@ class DpOnModel:
             if best[0] > comm_cost:
                 best = (comm_cost, res_list, pp_deg, mem_remain, mem_cost, vtp)
         return best
+
+    def fit(self, bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, print_=True, mbsz_dict=None):
+        """Same arguments and return value as the reference (dynamic_programming.py:515-565):
+        ``(min_comm_cost, min_res_list, min_pp_deg, min_mem_remain, min_mem_cost, min_vtp)``.
+        All pipeline degrees are prepared first and their DP instances solved in one device batch."""
+        ticket, dps = self.fit_begin(bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, mbsz_dict)
+        return self.fit_end(ticket, DPAlg.fit_many(dps), print_)
