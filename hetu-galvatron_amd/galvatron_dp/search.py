@@ -10,8 +10,10 @@ filters, same tie-breaking (first strictly better throughput wins) and the same
 task (optionally on a thread pool); here the DP instances of ALL tasks of a sweep are collected
 first and solved in one device batch, then every task is finished from its share of the results.
 
-Reading the profilers' files (search_engine.py:119-337) is not part of this module: the cost-model
-argument records are handed in (``set_cost_model_args``).
+The cost-model argument records come either from the profilers' files
+(``set_search_engine_info`` + ``initialize_search_engine``, search_engine.py:45-337; the reading
+itself is in profile_configs.py) or directly from the caller (``set_model`` +
+``set_cost_model_args``).
 """
 from __future__ import annotations
 
@@ -21,7 +23,7 @@ import os
 
 import numpy as np
 
-from . import cost_models
+from . import cost_models, profile_configs
 from .dynamic_programming import DPAlg, DpOnModel
 from .pp_utils import check_optimal_chunks, get_pp_stage_for_bsz, optimal_chunk_func_default
 
@@ -68,19 +70,98 @@ class SearchEngine:
         self.optimal_chunk_func = optimal_chunk_func_default
         self.model_name = None
         self.path = None
+        self.mem_path = None
+        self.time_path = None
         self.strategies = None
         self.results = None
         self.optimal = None
         self.solved_instances = 0
 
-    # ---- what the reference reads from files / sets up in set_cost_models (search_engine.py:45-337) ----
+    # ---- model, paths (search_engine.py:45-97) ---------------------------------------------------------
     def set_model(self, model_name, model_layer_configs, path=None):
         self.model_name = model_name
         self.path = path
+        self.set_model_layer_configs(model_layer_configs)
+
+    def set_search_engine_info(self, path, model_layer_configs, model_name):
+        """``path``: the model's directory (profiles in ``<path>/configs`` unless the arguments name
+        another place); ``model_layer_configs``: one {'hidden_size', 'layer_num', 'seq_len'} per layer
+        type."""
+        self.set_model_layer_configs(model_layer_configs)
+        self.path = path
+        self.model_name = model_name
+        self.memory_profiling_path()
+        self.time_profiling_path()
+
+    def set_path(self, path):
+        self.path = path
+
+    def set_model_name(self, name):
+        self.model_name = name
+
+    def set_model_layer_configs(self, model_layer_configs):
+        if model_layer_configs is None:
+            return
         self.hiddensize_list = [c['hidden_size'] for c in model_layer_configs]
         self.layernum_list = [c['layer_num'] for c in model_layer_configs]
         self.seqlen_list = [c['seq_len'] for c in model_layer_configs]
         self.num_layertype = len(self.layernum_list)
+
+    def _profile_path(self, given, stem):
+        assert self.model_name is not None, 'Should specify the model name!'
+        base = os.path.join(self.path, 'configs') if given is None else given
+        return os.path.join(base, '%s_%s_%s.json' % (stem, self.args.mixed_precision, self.model_name))
+
+    def memory_profiling_path(self):
+        if self.mem_path is None:
+            self.mem_path = self._profile_path(self.args.memory_profiling_path, 'memory_profiling')
+        return self.mem_path
+
+    def time_profiling_path(self):
+        if self.time_path is None:
+            self.time_path = self._profile_path(self.args.time_profiling_path, 'computation_profiling')
+        return self.time_path
+
+    # ---- profiles -> argument records (search_engine.py:99-337) ---------------------------------------
+    def initialize_search_engine(self):
+        self.generate_strategies()
+        self.get_profiled_model_configs()
+        self.get_profiled_hardware_configs()
+        self.set_cost_models()
+
+    def get_profiled_model_configs(self):
+        args = self.args
+        self.time_config = profile_configs.read_json_config(self.time_profiling_path())
+        self.memory_config = profile_configs.int_keys(profile_configs.read_json_config(self.memory_profiling_path()))
+        self.time_profiled_list, self.other_time_profiled_list = profile_configs.fit_layer_times(
+            self.time_config, args.time_profile_mode, self.num_layertype, self.seqlen_list)
+        (self.param_sizes, self.act_sizes, self.other_memory_pp_off,
+         self.other_memory_pp_on) = profile_configs.layer_memory(
+            self.memory_config, args.memory_profile_mode, args.sequence_parallel, self.num_layertype, self.seqlen_list)
+        return self.time_config, self.memory_config
+
+    def get_profiled_hardware_configs(self):
+        """Also rewrites the four path arguments to the files' full names, as the reference does."""
+        args = self.args
+        (args.allreduce_bandwidth_config_path, args.p2p_bandwidth_config_path, args.overlap_coe_path,
+         args.sp_time_path) = profile_configs.hardware_paths(args, self.path)
+        self.allreduce_bandwidth, self.allreduce_comm_coe = profile_configs.read_allreduce_bandwidth_config(
+            args.allreduce_bandwidth_config_path, gpu_num=args.gpu_num)
+        self.p2p_bandwidth, self.p2p_comm_coe = profile_configs.read_p2p_bandwidth_config(args.p2p_bandwidth_config_path)
+        self.overlap_coe = profile_configs.read_json_config(args.overlap_coe_path)['overlap_coe']
+        sp_config = profile_configs.read_json_config(args.sp_time_path)
+        self.sp_allreduce = profile_configs.remap_config(sp_config, "allreduce")
+        self.sp_all2all = profile_configs.remap_config(sp_config, "all2all")
+        return self.allreduce_bandwidth, self.p2p_bandwidth, self.overlap_coe, self.sp_allreduce, self.sp_all2all
+
+    def set_cost_models(self):
+        records = [profile_configs.cost_model_args(
+            self.args, (self.hiddensize_list[i], self.layernum_list[i], self.seqlen_list[i]), self.optimal_chunk_func,
+            self.param_sizes[i], self.act_sizes[i], self.other_memory_pp_off, self.other_memory_pp_on,
+            self.time_profiled_list[i], self.other_time_profiled_list[0], self.allreduce_comm_coe, self.p2p_comm_coe,
+            self.overlap_coe, self.sp_allreduce, self.sp_all2all) for i in range(self.num_layertype)]
+        (self.model_args_list, self.train_args_list, self.parallel_args_list, self.profile_model_args_list,
+         self.profile_hardware_args_list) = [list(column) for column in zip(*records)]
 
     def set_cost_model_args(self, model_args_list, train_args_list, parallel_args_list, profile_model_args_list,
                             profile_hardware_args_list, allreduce_comm_coe):
