@@ -485,11 +485,14 @@ class OtherTimeCostModel:
         for k in degrees:
             # activation collectives of the embedding / head, one per sequence length (cost_model.py:533-570)
             times = []
+            # message sizes of the largest degree stay readable on the object, as in the reference
+            self.per_tp_message_size, self.tp_message_size = [], []
             for seq_len in sequence_length_list:
                 if vsp != 0:
                     times.append(0)
                 elif self.sp_space == 'tp+sp':
                     size = mbsz * seq_len * model_args.hidden_size * word
+                    self.per_tp_message_size.append(size)
                     if k == 1:
                         times.append(0)
                     elif size in hw.allreduce_dict:
@@ -500,6 +503,7 @@ class OtherTimeCostModel:
                     dp = world_size // pp_deg // k
                     coe = _group_coe(hw.comm_coe_dict, k) if (k == 1 or dp == 1) else _group_coe(hw.comm_coe_dict, k, 0)
                     size = (k - 1) / k * (mbsz * seq_len * self.hidden_size / 1024 / 1024) * word
+                    self.tp_message_size.append(size)
                     times.append(size * coe)
             self.tp_time[k] = (sum(times) + times[-1]) if pp_deg == 1 else (times[0], times[-1])
 
