@@ -149,24 +149,35 @@ struct HostInst {
 
 struct Group {  // instances with the same S, sorted by L descending
     int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt;
+    int xcd_group = 1;        // consecutive block tasks handed to one XCD (whole tiles)
+    int slots = 0;            // workgroups per XCD, instance and layer of a fused launch
     int64_t max_ld;
     std::vector<int> active;  // active[l] = number of instances with L > l
-    std::vector<std::pair<int, int>> segments;  // fused launches: (first layer, layers), same active set
+    std::vector<int64_t> live_blocks;  // block tasks of layer l that carry arithmetic, over its instances
+    struct Segment { int first, layers; unsigned lds_bytes; };
+    std::vector<Segment> segments;  // fused launches: runs of layers with the same active set
     size_t off_sched, off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
 // Target-tile width: the one that pads S the least; of two that pad alike the wider one, which
-// issues fewer cost-row loads per relaxation (S = 88: eight blocks of 11 rather than eleven of 8).
-int pick_ts(int S)
+// issues fewer cost-row loads per relaxation (S = 88: eight blocks of 11 rather than eleven of 8;
+// S = 64: four of 16).  marks: only among the variants built with the argmin table.
+int pick_ts(int S, bool marks)
 {
-    int best = GDP_VARIANTS[0].ts;
-    size_t best_sp = align_up((size_t)S, (size_t)best);
-    for (int v = 1; v < GDP_NUM_VARIANTS; ++v) {
+    int best = 0;
+    size_t best_sp = 0;
+    for (int v = 0; v < GDP_NUM_VARIANTS; ++v) {
+        if (marks && !GDP_VARIANTS[v].marks) continue;
         const size_t sp = align_up((size_t)S, (size_t)GDP_VARIANTS[v].ts);
-        if (sp < best_sp || (sp == best_sp && GDP_VARIANTS[v].ts > best)) { best = GDP_VARIANTS[v].ts; best_sp = sp; }
+        if (best == 0 || sp < best_sp || (sp == best_sp && GDP_VARIANTS[v].ts > best)) {
+            best = GDP_VARIANTS[v].ts;
+            best_sp = sp;
+        }
     }
     return best;
 }
+
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
 int find_variant(int ts, int r)
 {
@@ -204,10 +215,12 @@ struct gdp_plan {
     int64_t spin_limit = 1 << 22; // polls a waiting wave makes before the launch is abandoned
     size_t off_zero = 0, zero_words = 0, off_abort = 0;
     int num_cu = 0;
+    size_t lds_per_cu = 0;
     bool can_fuse = true;    // cost buffers were laid out one per layer
     bool rezero = false;     // buffer 0 is overwritten during a run and must be zeroed before each
     bool fused_gave_up = false;  // a fused launch was abandoned and the plan switched to per-layer launches
     bool no_fallback = false;    // GDP_OPT_NO_FALLBACK: report that instead of switching (tests)
+    bool no_occupancy_cap = false;  // GALVATRON_DP_OCCUPANCY_CAP=0 (tuning aid)
     int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
@@ -344,7 +357,11 @@ size_t footprint(const gdp_problem *q)
     return sizeof(double) * ((size_t)q->L + 1) * ((size_t)q->S + 1) * ld;
 }
 
-int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
+// Internal return code: the costs-only layout (one cost buffer per layer) does not fit in device memory;
+// the caller starts over with force_marks, i.e. two cost buffers and the argmin table.
+constexpr int GDP_RETRY_WITH_MARKS = 1 << 20;
+
+int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks)
 {
     pl->n = n;
     GDP_HIP(hipGetDevice(&pl->device));
@@ -362,15 +379,31 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
+    if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) pl->no_occupancy_cap = atoi(e) == 0;
     if (const char *e = getenv("GALVATRON_DP_SPIN_LIMIT")) {
         const long long v = atoll(e);
         if (v >= 1) pl->spin_limit = v;
+    }
+    for (int i = 0; i < n; ++i) {
+        if (p[i]->flags & GDP_COMPUTE_ALL) pl->skip = false;
+        if ((p[i]->flags & GDP_KEEP_MARKS) && !marks_preset) pl->keep_marks = true;
+        if (p[i]->flags & GDP_EXPORT_MARK) pl->keep_marks = true;  // the table itself is asked for
+    }
+    for (int i = 0; i < n && !fused_preset; ++i) {  // an explicit request of the caller
+        if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
+        else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
+    }
+    if (force_marks) {
+        pl->keep_marks = true;
+        pl->fused = false;
+        fused_preset = true;
     }
     // ---- shapes -------------------------------------------------------------------------------
     {
         hipDeviceProp_t prop;
         GDP_HIP(hipGetDeviceProperties(&prop, pl->device));
         pl->num_cu = prop.multiProcessorCount;
+        pl->lds_per_cu = prop.maxSharedMemoryPerMultiProcessor;
     }
     std::vector<HostInst> inst((size_t)n);
     for (int i = 0; i < n; ++i) {
@@ -402,7 +435,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         // Register tile.  Width: least padding of S.  Height: the tallest whose first layer still
         // gives every resident wave at least two tasks, so that the stores of one task drain under
         // the arithmetic of the next; small problems get the shortest (most parallel) one.
-        const int ts = pick_ts(g.S);
+        const int ts = pick_ts(g.S, pl->keep_marks);
         const int ntb = (int)align_up((size_t)g.S, (size_t)ts) / ts;
         int best_r = 0;
         {
@@ -438,24 +471,19 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         for (int k = i; k < j; ++k)
             for (int l = 0; l < inst[(size_t)k].L; ++l) g.active[(size_t)l]++;
         g.nbt = (g.max_ntile * g.ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
+        // whole tiles per XCD turn: the fewest tiles whose wave tasks fill whole workgroups
+        g.xcd_group = GDP_WAVES_PER_BLOCK / gcd_int(g.ntb, GDP_WAVES_PER_BLOCK) * g.ntb / GDP_WAVES_PER_BLOCK;
+        g.slots = ((g.nbt + g.xcd_group - 1) / g.xcd_group + 7) / 8 * g.xcd_group;
         pl->max_L = std::max(pl->max_L, g.max_L);
         pl->groups.push_back(g);
         i = j;
     }
-    for (int i = 0; i < n; ++i) {
-        if (p[i]->flags & GDP_COMPUTE_ALL) pl->skip = false;
-        if ((p[i]->flags & GDP_KEEP_MARKS) && !marks_preset) pl->keep_marks = true;
-        if (p[i]->flags & GDP_EXPORT_MARK) pl->keep_marks = true;  // the table itself is asked for
-    }
-    for (int i = 0; i < n && !fused_preset; ++i) {  // an explicit request of the caller
-        if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
-        else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
-    }
     if (!fused_preset) {
-        // One launch for all layers pays off when a layer holds at least twice as many block tasks
-        // that carry arithmetic as the device holds blocks: then what a block waits for was finished a
-        // while ago, and its loads, stores and waits hide under the arithmetic of its neighbours.
-        // Below that the latency of signalling through memory shows, and a launch per layer is quicker.
+        // One launch for all layers pays off once a layer holds about two block tasks that carry
+        // arithmetic per CU (measured: 950 per layer, 0.48 ms against 0.58 ms; 128 per layer, 0.23 ms
+        // against 0.17 ms): the launch gaps and the ramp up and down of every layer go away, and layers
+        // overlap where their dependencies allow.  Below that a layer is over before signalling through
+        // memory has paid for itself, and a launch per layer is quicker.
         double first_layer = 0, all = 0, live = 0;
         std::vector<int32_t> band;
         for (const Group &g : pl->groups) {
@@ -467,7 +495,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
                 all += (double)h.L * h.V * (double)h.S * h.S;
             }
         }
-        pl->fused = first_layer * (all > 0 ? live / all : 1.0) >= 2.0 * pl->num_cu * 4;
+        pl->fused = first_layer * (all > 0 ? live / all : 1.0) >= 2.0 * pl->num_cu;
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -531,9 +559,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         if (e == hipSuccess) break;
         pl->dbase = nullptr;
         (void)hipGetLastError();
-        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && max_S <= GDP_MAX_S_MARKS) {
-            pl->fused = false;
-            pl->keep_marks = true;
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && !pl->keep_marks &&
+            max_S <= GDP_MAX_S_MARKS)
+            return GDP_RETRY_WITH_MARKS;  // tile widths and paddings differ with the table: start over
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && pl->keep_marks) {
+            pl->fused = false;            // table kept and all layers in one launch: drop the latter
             continue;
         }
         char buf[128];
@@ -612,6 +642,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         // the per-(instance, layer) records; entries of layers an instance does not have stay zero but for hi
         GdpDevLayer *lay = reinterpret_cast<GdpDevLayer *>(stage.data() + g.off_lay);
         sc->lay = reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay);
+        g.live_blocks.assign((size_t)g.max_L, 0);
         for (int k = 0; k < g.count; ++k) {
             const HostInst &h = inst[(size_t)(g.first + k)];
             const gdp_problem *q = p[h.orig];
@@ -633,13 +664,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
                 y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
                 y.lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
                 y.hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
+                if (y.hi >= y.lo)
+                    g.live_blocks[(size_t)l] += ((int64_t)(y.hi - y.lo + 1) * g.ntb + GDP_WAVES_PER_BLOCK - 1) /
+                                                GDP_WAVES_PER_BLOCK;
             }
         }
         sc->cnt = reinterpret_cast<int32_t *>(pl->dbase + g.off_cnt);
         sc->abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
         sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb;
-        sc->slots = (g.nbt + 7) / 8 + 2;
+        sc->group = g.xcd_group;
+        sc->slots = g.slots;
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
         for (int l = 0; l < g.max_L; ++l) act[l] = g.active[(size_t)l];
@@ -648,17 +683,31 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl)
         g.segments.clear();
         for (int l = 0; l < g.max_L; ++l) {
             if (!g.segments.empty() && g.active[(size_t)l] == g.active[(size_t)g.segments.back().first] &&
-                g.segments.back().second < 65535)
-                g.segments.back().second++;
+                g.segments.back().layers < 65535)
+                g.segments.back().layers++;
             else
-                g.segments.push_back({l, 1});
+                g.segments.push_back({l, 1, 0u});
         }
         while (g.segments.size() > 32) {
             size_t best = 1;
             for (size_t i = 1; i < g.segments.size(); ++i)
-                if (g.segments[i].second < g.segments[best].second) best = i;
-            g.segments[best - 1].second += g.segments[best].second;
+                if (g.segments[i].layers < g.segments[best].layers) best = i;
+            g.segments[best - 1].layers += g.segments[best].layers;
             g.segments.erase(g.segments.begin() + (long)best);
+        }
+        // Workgroups are dispatched in order, so the ones resident at any time are a window of
+        // consecutive ones.  A window wider than the arithmetic of one layer reaches into the next
+        // layer, whose workgroups can only wait, and they take the places of ones that could run on
+        // CUs that then sit idle.  Dynamic LDS that the kernel never touches holds the number of
+        // workgroups per CU to (arithmetic-carrying block tasks of an average layer) / CUs, between 3
+        // and the 8 that fit anyway.
+        for (auto &seg : g.segments) {
+            int64_t sum = 0;
+            for (int l = seg.first; l < seg.first + seg.layers; ++l) sum += g.live_blocks[(size_t)l];
+            const int64_t per_cu = std::max<int64_t>(3, sum / seg.layers / std::max(pl->num_cu, 1));
+            seg.lds_bytes = 0;
+            if (per_cu < 8 && pl->lds_per_cu >= 65536 && !pl->no_occupancy_cap)
+                seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
     GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));
@@ -705,13 +754,12 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
         GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
                                 pl->stream));
         for (const Group &g : pl->groups)
-            for (const auto &seg : g.segments) {  // (first layer, number of layers)
-                // per XCD and instance: an eighth each of the block tasks below, inside and above the band
-                const int grid_x = 8 * g.active[(size_t)seg.first] * ((g.nbt + 7) / 8 + 2);
+            for (const auto &seg : g.segments) {
+                const int grid_x = 8 * g.active[(size_t)seg.first] * g.slots;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
                 GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
                                                reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,
-                                               seg.first, seg.second, pl->stream));
+                                               seg.first, seg.layers, seg.lds_bytes, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
@@ -834,20 +882,23 @@ int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
         int rc = validate(p[i], i);
         if (rc != GDP_OK) return rc;
     }
-    gdp_plan *pl = new (std::nothrow) gdp_plan();
-    if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
-    int rc;
-    try {
-        rc = create(n, p, pl);
-    } catch (const std::bad_alloc &) {
-        rc = fail(GDP_E_NOMEM, "host allocation failed");
-    }
-    if (rc != GDP_OK) {
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        gdp_plan *pl = new (std::nothrow) gdp_plan();
+        if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
+        int rc;
+        try {
+            rc = create(n, p, pl, attempt == 1);
+        } catch (const std::bad_alloc &) {
+            rc = fail(GDP_E_NOMEM, "host allocation failed");
+        }
+        if (rc == GDP_OK) {
+            *out = pl;
+            return GDP_OK;
+        }
         destroy(pl);
-        return rc;
+        if (rc != GDP_RETRY_WITH_MARKS || attempt == 1) return rc == GDP_RETRY_WITH_MARKS ? fail(GDP_E_NOMEM, "device memory") : rc;
     }
-    *out = pl;
-    return GDP_OK;
+    return fail(GDP_E_NOMEM, "device memory");
 }
 
 int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing)

@@ -86,7 +86,8 @@ struct GdpSched {
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
     int32_t max_L, max_ntile, ntb;
-    int32_t slots;            // workgroups per XCD, instance and layer: ceil(block tasks / 8) + 2
+    int32_t group;            // consecutive block tasks that go to one XCD (whole tiles)
+    int32_t slots;            // workgroups per XCD, instance and layer: ceil(ceil(block tasks / group) / 8) * group
     int64_t spin_limit;       // polls before a waiting wave gives up
 };
 
@@ -104,12 +105,16 @@ struct GdpDevOut {
 };
 
 // Register tile of the relaxation kernel: TS target strategies x (64 lanes x R rows) per wavefront.
-// Variants of one width are listed tallest first.
+// Variants of one width are listed tallest first.  A wider tile issues fewer cost-row loads per
+// relaxation (one 512-byte load feeds 2*TS vector instructions); the 16-wide ones exist for the
+// costs-only relaxation alone: with the argmin tracked as well they would not fit the registers.
 struct GdpVariant {
     int ts, r;
+    bool marks;  // also built with the argmin table
 };
-static const GdpVariant GDP_VARIANTS[] = {{8, 4}, {8, 2}, {8, 1}, {11, 3}, {11, 2}, {11, 1}};
-#define GDP_NUM_VARIANTS 6
+static const GdpVariant GDP_VARIANTS[] = {{16, 3, false}, {16, 2, false}, {16, 1, false}, {8, 4, true}, {8, 2, true},
+                                          {8, 1, true},   {11, 3, true},  {11, 2, true},  {11, 1, true}};
+#define GDP_NUM_VARIANTS 9
 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
 // marks: track and store the argmin table (otherwise costs only).  lay: the group's table of
@@ -118,8 +123,9 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int
                             int SP, int layer, hipStream_t stream);
 // Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
+// lds_bytes: dynamic LDS per workgroup, unused by the kernel; it limits how many workgroups a CU holds.
 hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
-                                  int layers, hipStream_t stream);
+                                  int layers, unsigned lds_bytes, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
 // in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).

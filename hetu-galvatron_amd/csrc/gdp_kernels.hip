@@ -6,8 +6,16 @@
 // f_prev[u][.] with lanes running along u (coalesced, no per-target shift), and keeps a tile of
 // running minima in registers.  Scanning s' upward and replacing only on strict '<' is the
 // comparison sequence of std::min_element (csrc/dp_core.cpp:12-16,70), so ties go to the lowest
-// index with no cross-lane traffic.  Both additions are done per candidate, in the reference's
-// order, before the comparison; nothing is pre-added or reassociated.
+// index with no cross-lane traffic.
+//
+// Where the argmin is tracked, both additions are done per candidate, in the reference's order,
+// before the comparison.  Where only the cost is wanted, intra[s] is added once, after the minimum:
+//   min_{s'} fl(fl(f + inter) + intra)  ==  fl(min_{s'} fl(f + inter) + intra)
+// holds exactly, because rounding x -> fl(x + c) is monotone (x <= y implies fl(x+c) <= fl(y+c)), so
+// the smallest pre-sum yields the smallest candidate; +inf behaves the same on both sides and NaN
+// and -inf are rejected on the host.  (Which s' attains the minimum can differ between the two
+// sides when two candidates round to the same value; the argmin is therefore never taken from the
+// hoisted form.)
 #include "gdp_kernels.h"
 
 #include <math.h>
@@ -39,12 +47,28 @@ __device__ __forceinline__ unsigned xcd_swizzle(unsigned x, unsigned nblk)
     return (x & 7u) * (nblk >> 3) + (x >> 3);
 }
 
+// Element lane + 64 r of a wave-uniform row: uniform 64-bit base plus a 32-bit per-lane byte offset,
+// the form that needs no per-lane address arithmetic (scalar base register + vector offset).  The
+// callers pass the base through an empty asm, and the offset once per basic block (GDP_PIN_LANE), or
+// the compiler folds the per-lane part into a 64-bit vector base outside the loop and spends one
+// vector instruction per load on adding the row offset to it.
+__device__ __forceinline__ double lane_load(const double *row, unsigned lane_bytes, int r)
+{
+    typedef const __attribute__((address_space(1))) char *gbytes;     // global memory, not "flat"
+    typedef const __attribute__((address_space(1))) double *gdouble;
+    return *reinterpret_cast<gdouble>(reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(row)) + lane_bytes +
+                                      512u * (unsigned)r);
+}
+
+#define GDP_PIN_LANE(x) asm volatile("" : "+v"(x))
+
 // Nothing is moved across this point by the instruction scheduler.
 #define GDP_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// Relaxations of target columns [J0, J1) of the register tile against one source strategy:
-// candidate = (f_prev + inter) + intra in that association (csrc/dp_core.cpp:68), strict '<' for the
-// argmin (csrc/dp_core.cpp:12-16).
+// Relaxations of target columns [J0, J1) of the register tile against one source strategy.
+// ARG: candidate = (f_prev + inter) + intra in that association (csrc/dp_core.cpp:68), strict '<' for
+// the argmin (csrc/dp_core.cpp:12-16).  Otherwise: the running minimum of f_prev + inter; the caller
+// adds intra at the end.
 template <int TS, int R, bool ARG, int J0, int J1>
 __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG ? R : 1][ARG ? TS : 1],
                                            const double (&fp)[R], const double (&sc)[TS], const double (&add)[TS],
@@ -54,7 +78,7 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
     for (int j = J0; j < J1; ++j)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const double c = (fp[r] + sc[j]) + add[j];
+            const double c = ARG ? (fp[r] + sc[j]) + add[j] : fp[r] + sc[j];
             if constexpr (ARG) {
                 // compare into vcc and select at once: left to the compiler, the compare results of a
                 // whole step end up in as many scalar register pairs, which then spill
@@ -72,8 +96,9 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
 // PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
 // waits for this task's completion counter finds them in memory.
 // ARG: also track and store the argmin (the reference's mark table, csrc/dp_core.cpp:70-72).  Without
-// it a relaxation is two additions and one minimum; the backtrack then recomputes the argmin of the
-// few cells on its path from the cost buffers, all of which are kept in that mode.
+// it a relaxation is one addition and one minimum (intra is added once per cell, see the top of this
+// file); the backtrack then recomputes the argmin of the few cells on its path from the cost
+// buffers, all of which are kept in that mode.
 template <int TS, int R, bool PUBLISH, bool ARG>
 __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
 {
@@ -86,9 +111,11 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
     const double *ia = uload(&Y->ia) + s0;
     const int64_t u0 = (int64_t)tile * (64 * R);
 
+    const unsigned lane_bytes = lane * 8u;
+
     double add[TS];
 #pragma unroll
-    for (int j = 0; j < TS; ++j) add[j] = uload(ia + j);
+    for (int j = 0; j < TS; ++j) add[j] = ARG ? uload(ia + j) : 0.0;  // without ARG: fetched after the loop
 
     double best[R][TS];
     int arg[ARG ? R : 1][ARG ? TS : 1];
@@ -122,12 +149,15 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
 #pragma unroll
         for (int u = 0; u < NS; ++u) o0[u] = uload(ro + u);
         GDP_SCHED_FENCE();
+        unsigned lb = lane_bytes;
+        GDP_PIN_LANE(lb);
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
             const double *p = src + o0[u] + u0;
+            asm volatile("" : "+s"(p));   // stays a scalar base (see lane_load)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                fp[u][r] = p[lane + 64u * r];
+                fp[u][r] = lane_load(p, lb, r);
                 GDP_SCHED_FENCE();
             }
         }
@@ -136,6 +166,8 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
         GDP_SCHED_FENCE();
     }
     for (int sp = 0; sp < SU; sp += NS) {
+        unsigned lb = lane_bytes;
+        GDP_PIN_LANE(lb);
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
             relax_cols<TS, R, ARG, 0, 1>(best, arg, fp[u], sc[u & 1], add, sp + u);
@@ -149,8 +181,9 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
             GDP_SCHED_FENCE();
             {
                 const double *pn = src + off + u0;
+                asm volatile("" : "+s"(pn));
 #pragma unroll
-                for (int r = 0; r < R; ++r) fp[u][r] = pn[lane + 64u * r];
+                for (int r = 0; r < R; ++r) fp[u][r] = lane_load(pn, lb, r);
             }
             GDP_SCHED_FENCE();
             off = off_next;
@@ -163,6 +196,15 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
     // made before the loop.)
     const GdpDevLayer *Z = Y;
     asm volatile("" : "+s"(Z));
+    if constexpr (!ARG) {
+        const double *iz = uload(&Z->ia) + s0;
+#pragma unroll
+        for (int j = 0; j < TS; ++j) {
+            const double a = uload(iz + j);
+#pragma unroll
+            for (int r = 0; r < R; ++r) best[r][j] += a;
+        }
+    }
     const int64_t ld = uload(&Z->ld);
     const int nvalid = uload(&Z->S) - s0;  // target strategies of this block that exist (>= 1)
     double *drow = uload(&Z->dst) + (int64_t)s0 * ld + u0;
@@ -292,7 +334,23 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
                                            int32_t *abort_flag, int64_t limit)
 {
     int64_t polls = 0;
-    for (int base = lo; base <= hi; base += 64) {
+    // First a look at up to four lanes-wide chunks at once (one round trip instead of four when
+    // everything is ready, as it mostly is); the chunks that are not are polled one after the other.
+    int first_unready = lo;
+    {
+        int v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int t = lo + 64 * c + (int)lane;
+            v[c] = (t <= hi) ? ld_agent(cnt + t) : full;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (__builtin_amdgcn_ballot_w64(v[c] < full) != 0) break;
+            first_unready = lo + 64 * (c + 1);
+        }
+    }
+    for (int base = first_unready; base <= hi; base += 64) {
         const int t = base + (int)lane;
         for (;;) {
             const int v = (t <= hi) ? ld_agent(cnt + t) : full;
@@ -334,10 +392,7 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //    L2 cannot hold an older copy of those lines: tiles are whole cache lines, nobody reads a tile
 //    before its counter is full, and the caches are invalidated when the launch begins.
 //
-// Share of an XCD: of every instance, one contiguous eighth of the block tasks that carry
-// arithmetic (tiles lo..hi of the layer), one eighth of those below (filled with +inf) and one
-// eighth of those above (only counted as done), so that all XCDs carry the same load whatever the
-// bands are, and neighbouring budget rows of a layer and of the layer before it meet in one L2.
+// Share of an XCD: of every instance, every eighth group of block tasks (see below).
 template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
     const GdpSched *__restrict__ Q, int layer0)
@@ -352,9 +407,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned nat = (unsigned)uload(uload(&Q->n_active) + layer);
     const unsigned xcd = blockIdx.x & 7u;   // workgroups go to the XCDs round-robin by linear id;
     const unsigned pos = blockIdx.x >> 3;   // gridDim.x is a multiple of 8
-    // Instance-major: the workgroups that an XCD runs at the same time work on neighbouring tiles of
-    // a few instances, whose source rows overlap (a tile reads dep+1 tiles of the layer before), so
-    // that the overlap is fetched from HBM once and then found in this XCD's L2.
+    // Instance-major: the workgroups that an XCD runs at the same time work on a few instances only.
     const unsigned slots = (unsigned)uload(&Q->slots);
     const unsigned ii = pos / slots;        // instance (a prefix of the table is active)
     const unsigned w = pos - ii * slots;    // slot within the XCD's share of that instance
@@ -363,36 +416,20 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const int ntile = uload(&Y->ntile);
     const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     const int lo = uload(&Y->lo), hi = uload(&Y->hi);
-    unsigned bt_lo = 0, n_live = 0;
-    if (hi >= lo) {
-        bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
-        unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
-        if (bt_hi > nbt - 1u) bt_hi = nbt - 1u;
-        n_live = bt_hi - bt_lo + 1u;
-    }
-    // Order inside the XCD's share of an instance: the block tasks below the band first (they only
-    // store +inf, and the layer after this one waits for some of them), then the ones that carry
-    // arithmetic, then those above the band (nothing to do but to count as done).
-    const unsigned n_fill = bt_lo, n_dead = nbt - n_fill - n_live;
-    const unsigned per_fill = (n_fill + 7u) >> 3, per_live = (n_live + 7u) >> 3, per_dead = (n_dead + 7u) >> 3;
-    unsigned bt;
+    // Block tasks run over (tile, target block) in that order; groups of `group` consecutive ones
+    // (whole tiles) are dealt to the XCDs in turn, and every XCD takes its groups in ascending order.
+    // So all XCDs move up the budget rows of a layer side by side: whatever the band of the layer is,
+    // each carries an eighth of it, and what a block waits for -- tiles at and below its own in the
+    // layer before -- was handed out a whole layer earlier on every XCD.
+    const unsigned G = (unsigned)uload(&Q->group);
+    const unsigned grp = w / G;
+    const unsigned bt = (grp * 8u + xcd) * G + (w - grp * G);
+    if (bt >= nbt) return;
     bool live = false;
-    if (w < per_fill) {
-        const unsigned i = xcd * per_fill + w;
-        if (i >= n_fill) return;
-        bt = n_fill - 1u - i;  // from the band downwards: the lowest tiles of the next layer's band, which
-                               // XCD 0 computes, read the tiles just below this layer's band
-    } else if (w < per_fill + per_live) {
-        const unsigned i = xcd * per_live + (w - per_fill);
-        if (i >= n_live) return;
-        bt = bt_lo + i;
-        live = true;
-    } else {
-        const unsigned w2 = w - per_fill - per_live;
-        if (w2 >= per_dead) return;
-        const unsigned i = xcd * per_dead + w2;
-        if (i >= n_dead) return;
-        bt = bt_lo + n_live + i;
+    if (hi >= lo) {
+        const unsigned bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
+        const unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
+        live = bt >= bt_lo && bt <= bt_hi;   // carries arithmetic; the others only fill or count as done
     }
     int32_t *cnt_all = uload(&Q->cnt);
     const unsigned q0 = bt * GDP_WAVES_PER_BLOCK;
@@ -639,16 +676,44 @@ static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, 
     return hipGetLastError();
 }
 
-// one entry per element of GDP_VARIANTS, in the same order
-#define GDP_FOR_EACH_VARIANT(X) X(0, 8, 4) X(1, 8, 2) X(2, 8, 1) X(3, 11, 3) X(4, 11, 2) X(5, 11, 1)
+// one entry per element of GDP_VARIANTS, in the same order: (index, TS, R, built with the argmin table)
+#define GDP_FOR_EACH_VARIANT(X)                                                                          \
+    X(0, 16, 3, false) X(1, 16, 2, false) X(2, 16, 1, false) X(3, 8, 4, true) X(4, 8, 2, true) X(5, 8, 1, true) \
+    X(6, 11, 3, true) X(7, 11, 2, true) X(8, 11, 1, true)
+
+template <int TS, int R, bool MARKS_BUILT>
+static hipError_t launch_relax_v(bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile, int SP, int layer,
+                          hipStream_t stream)
+{
+    if constexpr (MARKS_BUILT) {
+        if (marks) return launch_relax_t<TS, R, true>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+    } else if (marks) {
+        return hipErrorInvalidValue;
+    }
+    return launch_relax_t<TS, R, false>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+}
+
+template <int TS, int R, bool MARKS_BUILT>
+static hipError_t launch_fused_v(bool marks, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
+                          const GdpSched *sched, int layer0)
+{
+    if constexpr (MARKS_BUILT) {
+        if (marks) {
+            hipLaunchKernelGGL((gdp_relax_fused_kernel<TS, R, true>), grid, block, lds_bytes, stream, sched, layer0);
+            return hipGetLastError();
+        }
+    } else if (marks) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL((gdp_relax_fused_kernel<TS, R, false>), grid, block, lds_bytes, stream, sched, layer0);
+    return hipGetLastError();
+}
 
 hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile,
                             int SP, int layer, hipStream_t stream)
 {
-#define X(id, ts, r)                                                                                  \
-    case id:                                                                                          \
-        return marks ? launch_relax_t<ts, r, true>(lay, max_L, n_inst, max_ntile, SP, layer, stream)  \
-                     : launch_relax_t<ts, r, false>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+#define X(id, ts, r, m) \
+    case id: return launch_relax_v<ts, r, m>(marks, lay, max_L, n_inst, max_ntile, SP, layer, stream);
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
@@ -657,22 +722,16 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int
 }
 
 hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
-                                  int layers, hipStream_t stream)
+                                  int layers, unsigned lds_bytes, hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
-#define X(id, ts, r)                                                                                              \
-    case id:                                                                                                      \
-        if (marks)                                                                                                \
-            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, true>), grid, block, 0, stream, sched, layer0);  \
-        else                                                                                                      \
-            hipLaunchKernelGGL((gdp_relax_fused_kernel<ts, r, false>), grid, block, 0, stream, sched, layer0); \
-        break;
+#define X(id, ts, r, m) \
+    case id: return launch_fused_v<ts, r, m>(marks, grid, block, lds_bytes, stream, sched, layer0);
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;
     }
 #undef X
-    return hipGetLastError();
 }
 
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)
