@@ -12,16 +12,21 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    both sides).  The timed solves carry out EVERY one of the L*V*S*S relaxations
                    (GDP_COMPUTE_ALL); ``with_row_skipping`` reports the library's default, which
                    skips rows it can prove irrelevant and returns identical results.
-* ``roofline``     for the relaxation kernel (the only kernel that matters): 3 fp64 vector
-                   operations (two additions, one comparison) per relaxation, divided by the average
-                   launch duration measured with HIP events on the stream the kernel runs on;
+* ``roofline``     for the relaxation kernel (the only kernel that matters): the ALGORITHMIC 3 fp64
+                   vector operations per relaxation (two additions and one comparison per candidate,
+                   as the reference's loop does them), divided by the average launch duration
+                   measured with HIP events on the stream the kernel runs on;
                    peak = 39.3 TFLOP/s = MI355X's published 78.6 TFLOP/s fp64 vector rate, which
                    counts an FMA as two operations -- additions and comparisons cannot fuse.
+                   The kernel itself issues fewer: one addition and one minimum per relaxation plus
+                   one addition per cell (intra is added after the minimum, which is exact because
+                   rounding is monotone); ``issued_ops_per_relaxation`` and ``frac_issued`` give the
+                   fraction of the peak in instructions actually issued.
                    ``roofline_hbm`` is the same launch against 8 TB/s with the algorithmic bytes
                    V*S*(8 read + 8 write) per layer and instance (the relaxation stores costs only;
                    the backtrack recomputes the argmin of the L cells on its path.  ``with_mark_table``
                    reports the mode that stores the reference's argmin table instead: 17 bytes and
-                   five instead of three vector instructions per relaxation).
+                   five instead of two vector instructions per relaxation).
 * ``cpu_baseline`` the reference's own dp_core (compiled into oracle/_ref by oracle/build.py) or,
                    where that file is absent, the C restatement in oracle/, timed on this host on a
                    bounded sample of the same workload (its first layers), one thread.
@@ -43,8 +48,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the relaxation kernel measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (scaled by a copy kernel of known size); see profiles/.  None until measured.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "cfg2": 10.916e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
-    "cfg3": 45.2e9,     # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
+    "cfg2": 12.131e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
+    "cfg3": 46.81e9,    # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
+    "cfg2+row_skipping": 8.641e9,   # profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt
 }
 
 
@@ -97,6 +103,12 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--row-skipping", action="store_true",
+                    help="time the library's default (rows that need no arithmetic are filled or left out) instead "
+                         "of carrying out every relaxation; the line says so and gives the executed fraction")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="leave out the row-skipping and mark-table legs (profiling runs: the trace then holds the "
+                         "headline's launches alone)")
     ap.add_argument("--also", default="cfg3", help="comma-separated extra workloads summarised in the same line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run three device-to-device copies of 1 GiB (a kernel of known traffic, to scale the "
@@ -153,16 +165,17 @@ def main() -> int:
             "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
             "device_ms": t1.total_ms, "executed_fraction": tm.executed / relax,
             "tflops": 3.0 * tm.executed / launches / avg_launch_s / 1e12,
+            "issued_per_relaxation": 5.0 if keep_marks else 2.0 + 1.0 / insts[0].S,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
             "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
             "kernel": "gdp_relax_fused_kernel" if tm.fused else "gdp_relax_kernel",
         }
 
-    m = measure(a.workload, a.steps, a.warmup)
+    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping)
     insts = m["insts"]
     first = insts[0]
-    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(a.workload)
+    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(a.workload + ("+row_skipping" if a.row_skipping else ""))
     line = {
         "metric": "min-plus relaxations/s (L*V*S^2)", "value": m["value"], "unit": "relaxations/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": m["ms_per_step"],
@@ -170,11 +183,13 @@ def main() -> int:
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
                    "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
-                   "device": _lib.device_info()},
+                   "relaxations_executed_fraction": m["executed_fraction"], "device": _lib.device_info()},
         "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
                      "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,
                      "kernel": m["kernel"], "launches_per_step": m["launches"],
-                     "avg_launch_ms": m["avg_launch_ms"], "flops_per_relaxation": 3},
+                     "avg_launch_ms": m["avg_launch_ms"], "flops_per_relaxation": 3,
+                     "issued_ops_per_relaxation": m["issued_per_relaxation"],
+                     "frac_issued": m["tflops"] / 3.0 * m["issued_per_relaxation"] / PEAK_FP64_VALU_TFLOPS},
         "roofline_hbm": {"bound": "hbm", "achieved": m["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": m["gbs"] / PEAK_HBM_GBS, "traffic": traffic,
                          "algorithmic_bytes_per_launch": m["bytes_per_launch"]},
@@ -188,16 +203,20 @@ def main() -> int:
                    "roofline_frac_hbm": mm["gbs"] / PEAK_HBM_GBS, "avg_launch_ms": mm["avg_launch_ms"]}
     if also:
         line["also"] = also
-    # The library's default additionally leaves out rows it can prove irrelevant (all-infinite sources /
-    # unreachable from every start row); results are identical, fewer relaxations are carried out.
-    ms = measure(a.workload, max(3, a.steps // 2), 1, compute_all=False)
-    line["with_row_skipping"] = {"value_nominal": ms["value"], "ms_per_step": ms["ms_per_step"],
-                                 "relaxations_executed_fraction": ms["executed_fraction"],
-                                 "roofline_frac_valu_fp64_executed": ms["tflops"] / PEAK_FP64_VALU_TFLOPS}
-    mk = measure(a.workload, max(3, a.steps // 2), 1, keep_marks=True)
-    line["with_mark_table"] = {"value": mk["value"], "ms_per_step": mk["ms_per_step"],
-                               "roofline_frac_valu_fp64": mk["tflops"] / PEAK_FP64_VALU_TFLOPS,
-                               "algorithmic_bytes_per_launch": mk["bytes_per_launch"]}
+    if a.row_skipping:
+        del line["roofline_hbm"]       # its algorithmic bytes are those of the full table
+        line["metric"] += " -- NOMINAL count over time with row skipping on; roofline figures count executed relaxations"
+    if not a.headline_only:
+        # The library's default additionally leaves out rows it can prove irrelevant (all-infinite sources /
+        # unreachable from every start row); results are identical, fewer relaxations are carried out.
+        ms = measure(a.workload, max(3, a.steps // 2), 1, compute_all=False)
+        line["with_row_skipping"] = {"value_nominal": ms["value"], "ms_per_step": ms["ms_per_step"],
+                                     "relaxations_executed_fraction": ms["executed_fraction"],
+                                     "roofline_frac_valu_fp64_executed": ms["tflops"] / PEAK_FP64_VALU_TFLOPS}
+        mk = measure(a.workload, max(3, a.steps // 2), 1, keep_marks=True)
+        line["with_mark_table"] = {"value": mk["value"], "ms_per_step": mk["ms_per_step"],
+                                   "roofline_frac_valu_fp64": mk["tflops"] / PEAK_FP64_VALU_TFLOPS,
+                                   "algorithmic_bytes_per_launch": mk["bytes_per_launch"]}
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(a.workload)
     print(json.dumps(line))

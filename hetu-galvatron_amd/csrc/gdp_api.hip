@@ -471,7 +471,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         for (int k = i; k < j; ++k)
             for (int l = 0; l < inst[(size_t)k].L; ++l) g.active[(size_t)l]++;
         g.nbt = (g.max_ntile * g.ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
-        // whole tiles per XCD turn: the fewest tiles whose wave tasks fill whole workgroups
+        // Whole tiles per XCD turn: the fewest whose wave tasks fill whole workgroups.  (Longer turns
+        // would save some of the cache lines that neighbouring tiles share -- a tile's source rows start
+        // at any 8-byte offset -- from being fetched into two L2s, but measured slower: cfg3 49.5 ms with
+        // one tile per turn, 50.7 with two or four, 54 with eight.)
         g.xcd_group = GDP_WAVES_PER_BLOCK / gcd_int(g.ntb, GDP_WAVES_PER_BLOCK) * g.ntb / GDP_WAVES_PER_BLOCK;
         g.slots = ((g.nbt + g.xcd_group - 1) / g.xcd_group + 7) / 8 * g.xcd_group;
         pl->max_L = std::max(pl->max_L, g.max_L);

@@ -60,6 +60,33 @@ def test_random_instances_against_oracle(n, shape):
         _compare(inst, f"shape {shape} variant {variant}", launch=("fused", "per_layer", None, None)[variant])
 
 
+@pytest.mark.parametrize("shape", [(4, 8, 300), (3, 16, 200), (5, 11, 257), (3, 64, 150), (2, 44, 129)])
+def test_candidates_that_collide_only_after_the_intra_addition(shape):
+    """Transition costs that differ in the last bits under intra costs some 2^40 times larger: many
+    candidates (f + inter) + intra are then EQUAL although their (f + inter) differ, so the reference's
+    lowest-index rule picks a source that is not the one with the smallest f + inter.  The costs-only
+    relaxation takes the minimum before adding intra (the cost is the same, rounding being monotone);
+    the strategies must still be the reference's, in both modes and both launch schemes."""
+    L, S, V = shape
+    rng = np.random.Generator(np.random.PCG64([91, L, S, V]))
+    inst = W.random_instance(rng, L, S, V, mem_hi=max(1, V // (L + 1)), per_layer_inter=True, n_keys=3)
+    inst.inter_tables[...] = 1.0 + rng.integers(0, 6, size=inst.inter_tables.shape) * 2.0 ** -50
+    inst.inter[...] = inst.inter_tables[inst.inter_index]
+    inst.intra[...] = 2.0 ** 20 * rng.integers(1, 4, size=inst.intra.shape)
+    wt, wr, wm, wf, wmark = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+    # the scenario does what it is meant to: some cell's reference argmin is not its argmin of f + inter
+    f0 = np.zeros((V, S))
+    differs = 0
+    for v in range(V):
+        for s in range(S):
+            if v >= inst.mem[0][s]:
+                pre = f0[v - inst.mem[0][s]] + inst.inter[0][:, s]
+                differs += int(np.argmin(pre)) != int(wmark[0][v][s])
+    assert differs > 0
+    for launch in ("fused", "per_layer"):
+        _compare(inst, f"collisions {shape} {launch}", launch=launch)
+
+
 def test_no_keys_and_single_layer():
     rng = np.random.Generator(np.random.PCG64(5))
     inst = W.random_instance(rng, 1, 6, 50, mem_hi=20)
