@@ -89,6 +89,11 @@ void arena_trim(int device /* -1: every device */)
 // The smallest kept allocation of `device` that holds `need` bytes, or a fresh one.
 hipError_t arena_take(int device, size_t need, char **ptr, size_t *bytes)
 {
+    // test aid: requests above GALVATRON_DP_DEVICE_LIMIT_MB are answered like a device that is full
+    if (getenv("GALVATRON_DP_DEVICE_LIMIT_MB") && need > env_mb("GALVATRON_DP_DEVICE_LIMIT_MB", 0)) {
+        *ptr = nullptr;
+        return hipErrorOutOfMemory;
+    }
     {
         std::lock_guard<std::mutex> lk(g_arena_mu);
         size_t best = g_arenas.size();

@@ -135,6 +135,31 @@ def test_batch_solved_in_parts_and_allocation_reuse(golden, monkeypatch):
         _check_against_golden(prob, golden[n], n)
 
 
+def test_device_memory_short_for_one_buffer_per_layer(golden, monkeypatch):
+    """A device too full for one cost buffer per layer: plan creation starts over with two cost
+    buffers and the argmin table (and the register tiles that exist for that mode; S = 64 uses a
+    16-wide tile otherwise), with the same results; too full for that as well: MemoryError.  The
+    shortage is forced from the host (allocation requests above a limit are refused)."""
+    rec = golden["cfg2_small"]                         # L=12, S=64, V=12288: ~90 MB against ~25 MB
+    inst = H.build_case(rec)
+    _lib.cache_trim()
+    monkeypatch.setenv("GALVATRON_DP_DEVICE_LIMIT_MB", "48")
+    prob = _problem(inst, export_f=True)
+    with _lib.Plan([prob]) as plan:
+        t = plan.run(1)
+        plan.fetch()
+    _check_against_golden(prob, rec, "cfg2_small under a 48 MB limit")
+    assert H.sha(prob.f_out) == rec["f_sha256"]
+    assert t.relax_bytes == float(inst.L) * inst.V * inst.S * 17 and not t.fused
+    monkeypatch.setenv("GALVATRON_DP_DEVICE_LIMIT_MB", "4")
+    with pytest.raises(MemoryError):
+        _lib.solve_batch([_problem(inst)])
+    monkeypatch.delenv("GALVATRON_DP_DEVICE_LIMIT_MB")
+    prob = _problem(inst)
+    _lib.solve_batch([prob])
+    _check_against_golden(prob, rec, "cfg2_small afterwards")
+
+
 def test_abandoned_fused_launch_falls_back_or_reports(golden):
     """A spin limit of 1 makes waiting wavefronts give up at once (forced from the host; every
     kernel still runs to completion).  With the fallback the plan switches to per-layer launches
