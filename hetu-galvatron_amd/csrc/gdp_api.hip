@@ -226,6 +226,7 @@ struct gdp_plan {
     bool fused_gave_up = false;  // a fused launch was abandoned and the plan switched to per-layer launches
     bool no_fallback = false;    // GDP_OPT_NO_FALLBACK: report that instead of switching (tests)
     bool no_occupancy_cap = false;  // GALVATRON_DP_OCCUPANCY_CAP=0 (tuning aid)
+    int occupancy_cap_override = 0; // GALVATRON_DP_OCCUPANCY_CAP=n: n workgroups per CU in fused launches
     int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
@@ -384,7 +385,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
-    if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) pl->no_occupancy_cap = atoi(e) == 0;
+    if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) {
+        pl->no_occupancy_cap = atoi(e) == 0;
+        pl->occupancy_cap_override = atoi(e);
+    }
     if (const char *e = getenv("GALVATRON_DP_SPIN_LIMIT")) {
         const long long v = atoll(e);
         if (v >= 1) pl->spin_limit = v;
@@ -712,7 +716,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         for (auto &seg : g.segments) {
             int64_t sum = 0;
             for (int l = seg.first; l < seg.first + seg.layers; ++l) sum += g.live_blocks[(size_t)l];
-            const int64_t per_cu = std::max<int64_t>(3, sum / seg.layers / std::max(pl->num_cu, 1));
+            int64_t per_cu = std::max<int64_t>(3, sum / seg.layers / std::max(pl->num_cu, 1));
+            if (pl->occupancy_cap_override >= 3) per_cu = pl->occupancy_cap_override;
             seg.lds_bytes = 0;
             if (per_cu < 8 && pl->lds_per_cu >= 65536 && !pl->no_occupancy_cap)
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
