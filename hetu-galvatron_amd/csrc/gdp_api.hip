@@ -160,7 +160,11 @@ struct Group {  // instances with the same S, sorted by L descending
     std::vector<int> active;  // active[l] = number of instances with L > l
     std::vector<int64_t> live_blocks;  // block tasks of layer l that carry arithmetic, over its instances
     struct Segment { int first, layers; unsigned lds_bytes; };
-    std::vector<Segment> segments;  // fused launches: runs of layers with the same active set
+    std::vector<Segment> segments;  // fused launches: runs of layers with the same active set, or -- chunked --
+                                    // runs of at most 65535 entries of the row table
+    int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
+    std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
+    size_t off_rows = 0;
     size_t off_sched, off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
@@ -227,6 +231,7 @@ struct gdp_plan {
     bool no_fallback = false;    // GDP_OPT_NO_FALLBACK: report that instead of switching (tests)
     bool no_occupancy_cap = false;  // GALVATRON_DP_OCCUPANCY_CAP=0 (tuning aid)
     int occupancy_cap_override = 0; // GALVATRON_DP_OCCUPANCY_CAP=n: n workgroups per CU in fused launches
+    int chunk_override = 0;         // GALVATRON_DP_CHUNK=n: n instances at a time in fused launches
     int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
@@ -385,6 +390,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
+    if (const char *e = getenv("GALVATRON_DP_CHUNK")) pl->chunk_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) {
         pl->no_occupancy_cap = atoi(e) == 0;
         pl->occupancy_cap_override = atoi(e);
@@ -446,14 +452,29 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // the arithmetic of the next; small problems get the shortest (most parallel) one.
         const int ts = pick_ts(g.S, pl->keep_marks);
         const int ntb = (int)align_up((size_t)g.S, (size_t)ts) / ts;
+        // A fused launch takes `chunk` instances at a time through all their layers (in the sorted
+        // order, so mostly instances of one depth): as many as keep two cost buffers each -- the layer
+        // being read and the one being written -- within GALVATRON_DP_CHUNK_MB (default 128) of the
+        // 256 MB memory-side cache.  With all instances of a batch layer by layer instead, a layer's
+        // output has long left that cache when the next layer reads it (256 instances of 24 MB per
+        // layer: 46.9 ms; two at a time: 42.0 ms).
+        {
+            size_t pair = 0;  // bytes of two cost buffers of the largest instance
+            for (int k = i; k < j; ++k)
+                pair = std::max(pair, 2 * sizeof(double) * ((size_t)g.S + 1) *
+                                          ((size_t)inst[(size_t)k].V + (size_t)inst[(size_t)k].P));
+            const size_t budget = env_mb("GALVATRON_DP_CHUNK_MB", 128);
+            g.chunk = (int)std::min<size_t>((size_t)g.count, std::max<size_t>(1, budget / std::max<size_t>(pair, 1)));
+            if (pl->chunk_override > 0) g.chunk = std::min(g.count, pl->chunk_override);
+        }
         int best_r = 0;
         {
             // variants of one width are listed tallest first
             for (int v = 0; v < GDP_NUM_VARIANTS; ++v) {
                 if (GDP_VARIANTS[v].ts != ts) continue;
                 const int r = GDP_VARIANTS[v].r;
-                int64_t tasks = 0;
-                for (int k = i; k < j; ++k) tasks += ((int64_t)inst[(size_t)k].V + 64 * r - 1) / (64 * r) * ntb;
+                int64_t tasks = 0;  // of the instances that are in flight together
+                for (int k = i; k < i + g.chunk; ++k) tasks += ((int64_t)inst[(size_t)k].V + 64 * r - 1) / (64 * r) * ntb;
                 best_r = r;
                 if (tasks >= 2 * wave_slots) break;
             }
@@ -530,6 +551,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         g.off_sched = take(sizeof(GdpSched));
         g.off_active = take(sizeof(int32_t) * (size_t)g.max_L);
         g.off_lay = take(sizeof(GdpDevLayer) * (size_t)g.count * (size_t)g.max_L);
+        g.rows.clear();
+        if (g.chunk < g.count)
+            for (int i0 = 0; i0 < g.count; i0 += g.chunk) {
+                const int cnt = std::min(g.chunk, g.count - i0);
+                for (int l = 0; l < inst[(size_t)(g.first + i0)].L; ++l) {  // the deepest of a chunk comes first
+                    g.rows.push_back(i0);
+                    g.rows.push_back(cnt);
+                    g.rows.push_back(l);
+                }
+            }
+        g.off_rows = take(sizeof(int32_t) * std::max<size_t>(g.rows.size(), 1));
     }
     for (auto &h : inst) {
         h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_PAD) * h.SP);
@@ -690,10 +722,19 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
         for (int l = 0; l < g.max_L; ++l) act[l] = g.active[(size_t)l];
-        // One fused launch per run of layers with the same number of active instances (grid.y <= 65535);
-        // a batch with very many different depths merges the shortest runs into their predecessors.
+        sc->rows = nullptr;
         g.segments.clear();
-        for (int l = 0; l < g.max_L; ++l) {
+        if (!g.rows.empty()) {
+            // chunked: the grid rows follow the table, at most 65535 per launch
+            memcpy(stage.data() + g.off_rows, g.rows.data(), sizeof(int32_t) * g.rows.size());
+            sc->rows = reinterpret_cast<const int32_t *>(pl->dbase + g.off_rows);
+            const int n_rows = (int)(g.rows.size() / 3);
+            for (int r0 = 0; r0 < n_rows; r0 += 65535) g.segments.push_back({r0, std::min(65535, n_rows - r0), 0u});
+        }
+        // Otherwise one fused launch per run of layers with the same number of active instances
+        // (grid.y <= 65535); a batch with very many different depths merges the shortest runs into
+        // their predecessors.
+        for (int l = 0; l < g.max_L && g.rows.empty(); ++l) {
             if (!g.segments.empty() && g.active[(size_t)l] == g.active[(size_t)g.segments.back().first] &&
                 g.segments.back().layers < 65535)
                 g.segments.back().layers++;
@@ -714,9 +755,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // workgroups per CU to (arithmetic-carrying block tasks of an average layer) / CUs, between 3
         // and the 8 that fit anyway.
         for (auto &seg : g.segments) {
-            int64_t sum = 0;
-            for (int l = seg.first; l < seg.first + seg.layers; ++l) sum += g.live_blocks[(size_t)l];
-            int64_t per_cu = std::max<int64_t>(3, sum / seg.layers / std::max(pl->num_cu, 1));
+            int64_t sum = 0, grid_rows = seg.layers;
+            if (g.rows.empty()) {
+                for (int l = seg.first; l < seg.first + seg.layers; ++l) sum += g.live_blocks[(size_t)l];
+            } else {  // an average grid row: `chunk` instances of an average (instance, layer)
+                int64_t pairs = 0;
+                for (int l = 0; l < g.max_L; ++l) { sum += g.live_blocks[(size_t)l]; pairs += g.active[(size_t)l]; }
+                sum = sum * g.chunk / std::max<int64_t>(pairs, 1);
+                grid_rows = 1;
+            }
+            int64_t per_cu = std::max<int64_t>(3, sum / grid_rows / std::max(pl->num_cu, 1));
             if (pl->occupancy_cap_override >= 3) per_cu = pl->occupancy_cap_override;
             seg.lds_bytes = 0;
             if (per_cu < 8 && pl->lds_per_cu >= 65536 && !pl->no_occupancy_cap)
@@ -768,7 +816,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                                 pl->stream));
         for (const Group &g : pl->groups)
             for (const auto &seg : g.segments) {
-                const int grid_x = 8 * g.active[(size_t)seg.first] * g.slots;
+                const int grid_x = 8 * (g.rows.empty() ? g.active[(size_t)seg.first] : g.chunk) * g.slots;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
                 GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
                                                reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,

@@ -86,6 +86,8 @@ struct GdpSched {
     int32_t *abort_flag;      // set when a bounded wait ran out                   (zeroed per run)
     const int32_t *n_active;  // [max_L] instances that still have layer l (a prefix of the table)
     int32_t max_L, max_ntile, ntb;
+    const int32_t *rows;      // per grid row (blockIdx.y) of a chunked launch: {first instance, instances, layer};
+                              // null: grid row y is layer layer0+y of the first n_active[layer] instances
     int32_t group;            // consecutive block tasks that go to one XCD (whole tiles)
     int32_t slots;            // workgroups per XCD, instance and layer: ceil(ceil(block tasks / group) / 8) * group
     int64_t spin_limit;       // polls before a waiting wave gives up
@@ -124,6 +126,7 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int
 // Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
 // lds_bytes: dynamic LDS per workgroup, unused by the kernel; it limits how many workgroups a CU holds.
+// With sched->rows set, layer0 is the first entry of that table and `layers` the number of entries.
 hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);

@@ -400,7 +400,19 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     __shared__ int sh_ok;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned lane = threadIdx.x & 63u;
-    const int layer = layer0 + (int)blockIdx.y;
+    // What this grid row is: layer layer0+y of all instances that have it, or -- chunked launch -- one
+    // layer of a few consecutive instances.  Grid rows are dispatched in order, so a chunked launch
+    // takes a few instances through ALL their layers before it turns to the next few: what a layer
+    // wrote is then still in the memory-side cache when the next layer reads it.
+    const int32_t *rows = uload(&Q->rows);
+    int layer = layer0 + (int)blockIdx.y;
+    unsigned first_inst = 0, n_inst = ~0u;
+    if (rows) {
+        const int32_t *row = rows + 3 * (int64_t)(layer0 + (int)blockIdx.y);
+        first_inst = (unsigned)uload(row);
+        n_inst = (unsigned)uload(row + 1);
+        layer = uload(row + 2);
+    }
     const int max_L = uload(&Q->max_L);
     const int max_ntile = uload(&Q->max_ntile);
     const unsigned ntb = (unsigned)uload(&Q->ntb);
@@ -409,9 +421,10 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned pos = blockIdx.x >> 3;   // gridDim.x is a multiple of 8
     // Instance-major: the workgroups that an XCD runs at the same time work on a few instances only.
     const unsigned slots = (unsigned)uload(&Q->slots);
-    const unsigned ii = pos / slots;        // instance (a prefix of the table is active)
-    const unsigned w = pos - ii * slots;    // slot within the XCD's share of that instance
-    if (ii >= nat) return;
+    const unsigned k = pos / slots;         // instance within the grid row
+    const unsigned ii = first_inst + k;     // instance (a prefix of the table has this layer)
+    const unsigned w = pos - k * slots;     // slot within the XCD's share of that instance
+    if (k >= n_inst || ii >= nat) return;
     const GdpDevLayer *Y = uload(&Q->lay) + ((int64_t)ii * max_L + layer);
     const int ntile = uload(&Y->ntile);
     const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
