@@ -45,11 +45,12 @@ sys.path.insert(0, os.path.join(ROOT, "hetu-galvatron_amd"))
 
 PEAK_FP64_VALU_TFLOPS = 39.3   # 78.6 TFLOP/s published (FMA = 2 ops) / 2
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the relaxation kernel measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE (scaled by a copy kernel of known size); see profiles/.  None until measured.
+# Bytes per launch of the relaxation kernel between the L2s and the fabric (HBM and the memory-side
+# cache in front of it), measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a copy
+# kernel of known size; see profiles/.  None where not measured.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "cfg2": 12.131e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
-    "cfg3": 46.81e9,    # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
+    "cfg3": 199.6e9,    # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 177.2e9; one launch per solve)
     "cfg2+row_skipping": 8.641e9,   # profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt
 }
 
