@@ -681,6 +681,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->relaxations += (double)h.L * h.V * (double)h.S * h.S;
         pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + (pl->keep_marks ? 1 : 0));
     }
+    // grid.y of a launch; GALVATRON_DP_MAX_GRID_ROWS lowers it (test aid: splits launches of small cases)
+    int max_grid_rows = 65535;
+    if (const char *e = getenv("GALVATRON_DP_MAX_GRID_ROWS")) max_grid_rows = std::min(65535, std::max(1, atoi(e)));
     for (auto &g : pl->groups) {
         GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
         // the per-(instance, layer) records; entries of layers an instance does not have stay zero but for hi
@@ -729,14 +732,15 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             memcpy(stage.data() + g.off_rows, g.rows.data(), sizeof(int32_t) * g.rows.size());
             sc->rows = reinterpret_cast<const int32_t *>(pl->dbase + g.off_rows);
             const int n_rows = (int)(g.rows.size() / 3);
-            for (int r0 = 0; r0 < n_rows; r0 += 65535) g.segments.push_back({r0, std::min(65535, n_rows - r0), 0u});
+            for (int r0 = 0; r0 < n_rows; r0 += max_grid_rows)
+                g.segments.push_back({r0, std::min(max_grid_rows, n_rows - r0), 0u});
         }
         // Otherwise one fused launch per run of layers with the same number of active instances
         // (grid.y <= 65535); a batch with very many different depths merges the shortest runs into
         // their predecessors.
         for (int l = 0; l < g.max_L && g.rows.empty(); ++l) {
             if (!g.segments.empty() && g.active[(size_t)l] == g.active[(size_t)g.segments.back().first] &&
-                g.segments.back().layers < 65535)
+                g.segments.back().layers < max_grid_rows)
                 g.segments.back().layers++;
             else
                 g.segments.push_back({l, 1, 0u});

@@ -135,6 +135,29 @@ def test_batch_solved_in_parts_and_allocation_reuse(golden, monkeypatch):
         _check_against_golden(prob, golden[n], n)
 
 
+@pytest.mark.parametrize("chunk,max_rows", [(1, 65535), (3, 65535), (2, 5), (1000, 3), (4, 1)])
+def test_instances_taken_through_the_launch_a_few_at_a_time(golden, monkeypatch, chunk, max_rows):
+    """A fused launch takes `chunk` instances at a time through all their layers (grid rows follow a
+    table; more rows than a grid holds are split over launches -- forced here with a tiny limit).
+    Mixed depths, widths and budgets in one batch; chunk sizes that do and do not divide the groups."""
+    names = ["cfg3_smallV_%d" % i for i in range(8)] + ["ties_6", "rand_6", "infeasible_6", "ties_2", "cfg2_small",
+                                                        "rand_2", "infeasible_2"]
+    insts = [H.build_case(golden[n]) for n in names]
+    monkeypatch.setenv("GALVATRON_DP_CHUNK", str(chunk))
+    monkeypatch.setenv("GALVATRON_DP_MAX_GRID_ROWS", str(max_rows))
+    probs = [_problem(i, launch="fused") for i in insts]
+    with _lib.Plan(probs) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)
+        for _ in range(2):
+            t = plan.run(1)
+            plan.fetch()
+            for n, prob in zip(names, probs):
+                _check_against_golden(prob, golden[n], f"{n} chunk={chunk} rows={max_rows}")
+    assert t.fused
+    if max_rows < 10:
+        assert t.relax_launches > 4
+
+
 def test_device_memory_short_for_one_buffer_per_layer(golden, monkeypatch):
     """A device too full for one cost buffer per layer: plan creation starts over with two cost
     buffers and the argmin table (and the register tiles that exist for that mode; S = 64 uses a
