@@ -165,7 +165,8 @@ struct Group {  // instances with the same S, sorted by L descending
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
     std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
     size_t off_rows = 0;
-    size_t off_sched, off_active, off_cnt, off_lay;  // byte offsets in the device allocation
+    GdpSched sched = {};      // argument of the fused launches (device pointers inside)
+    size_t off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
 // Target-tile width: the one that pads S the least; of two that pad alike the wider one, which
@@ -548,7 +549,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     pl->off_insts = take(sizeof(GdpDevInst) * (size_t)n);
     pl->off_keys = take(sizeof(GdpDevKey) * (size_t)std::max(nk, 1));
     for (auto &g : pl->groups) {
-        g.off_sched = take(sizeof(GdpSched));
         g.off_active = take(sizeof(int32_t) * (size_t)g.max_L);
         g.off_lay = take(sizeof(GdpDevLayer) * (size_t)g.count * (size_t)g.max_L);
         g.rows.clear();
@@ -685,7 +685,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     int max_grid_rows = 65535;
     if (const char *e = getenv("GALVATRON_DP_MAX_GRID_ROWS")) max_grid_rows = std::min(65535, std::max(1, atoi(e)));
     for (auto &g : pl->groups) {
-        GdpSched *sc = reinterpret_cast<GdpSched *>(stage.data() + g.off_sched);
+        GdpSched *sc = &g.sched;
         // the per-(instance, layer) records; entries of layers an instance does not have stay zero but for hi
         GdpDevLayer *lay = reinterpret_cast<GdpDevLayer *>(stage.data() + g.off_lay);
         sc->lay = reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay);
@@ -823,7 +823,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                 const int grid_x = 8 * (g.rows.empty() ? g.active[(size_t)seg.first] : g.chunk) * g.slots;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
                 GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
-                                               reinterpret_cast<const GdpSched *>(pl->dbase + g.off_sched), grid_x,
+                                               g.sched, grid_x,
                                                seg.first, seg.layers, seg.lds_bytes, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
@@ -1000,10 +1000,7 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
             if (value < 1) return fail(GDP_E_BADARG, "spin limit must be >= 1");
             plan->spin_limit = value;
             GDP_HIP(hipSetDevice(plan->device));
-            for (const Group &g : plan->groups) {  // patch the device copies
-                GdpSched *sc = reinterpret_cast<GdpSched *>(plan->dbase + g.off_sched);
-                GDP_HIP(hipMemcpy(&sc->spin_limit, &value, sizeof value, hipMemcpyHostToDevice));
-            }
+            for (Group &g : plan->groups) g.sched.spin_limit = value;
             return GDP_OK;
         }
         default:

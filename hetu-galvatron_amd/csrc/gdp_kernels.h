@@ -79,7 +79,9 @@ struct GdpDevLayer {
 };
 static_assert(sizeof(GdpDevLayer) == 128, "one record = two 64-byte scalar loads");
 
-// Bookkeeping of one fused (all layers) launch over a group of instances.
+// Bookkeeping of one fused (all layers) launch over a group of instances.  Passed to the kernel by
+// value: its fields arrive with the kernel arguments, one dependent load fewer at the start of every
+// workgroup.
 struct GdpSched {
     const GdpDevLayer *lay;   // [n_inst][max_L]
     int32_t *cnt;             // [n_inst][max_L][max_ntile] finished wave tasks    (zeroed per run)
@@ -127,7 +129,7 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
 // lds_bytes: dynamic LDS per workgroup, unused by the kernel; it limits how many workgroups a CU holds.
 // With sched->rows set, layer0 is the first entry of that table and `layers` the number of entries.
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN

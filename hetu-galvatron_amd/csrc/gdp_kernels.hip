@@ -395,7 +395,7 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 // Share of an XCD: of every instance, every eighth group of block tasks (see below).
 template <int TS, int R, bool ARG>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
-    const GdpSched *__restrict__ Q, int layer0)
+    const GdpSched Q, int layer0)
 {
     __shared__ int sh_ok;
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     // layer of a few consecutive instances.  Grid rows are dispatched in order, so a chunked launch
     // takes a few instances through ALL their layers before it turns to the next few: what a layer
     // wrote is then still in the memory-side cache when the next layer reads it.
-    const int32_t *rows = uload(&Q->rows);
+    const int32_t *rows = Q.rows;
     int layer = layer0 + (int)blockIdx.y;
     unsigned first_inst = 0, n_inst = ~0u;
     if (rows) {
@@ -413,19 +413,19 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         n_inst = (unsigned)uload(row + 1);
         layer = uload(row + 2);
     }
-    const int max_L = uload(&Q->max_L);
-    const int max_ntile = uload(&Q->max_ntile);
-    const unsigned ntb = (unsigned)uload(&Q->ntb);
-    const unsigned nat = (unsigned)uload(uload(&Q->n_active) + layer);
+    const int max_L = Q.max_L;
+    const int max_ntile = Q.max_ntile;
+    const unsigned ntb = (unsigned)Q.ntb;
+    const unsigned nat = (unsigned)uload(Q.n_active + layer);
     const unsigned xcd = blockIdx.x & 7u;   // workgroups go to the XCDs round-robin by linear id;
     const unsigned pos = blockIdx.x >> 3;   // gridDim.x is a multiple of 8
     // Instance-major: the workgroups that an XCD runs at the same time work on a few instances only.
-    const unsigned slots = (unsigned)uload(&Q->slots);
+    const unsigned slots = (unsigned)Q.slots;
     const unsigned k = pos / slots;         // instance within the grid row
     const unsigned ii = first_inst + k;     // instance (a prefix of the table has this layer)
     const unsigned w = pos - k * slots;     // slot within the XCD's share of that instance
     if (k >= n_inst || ii >= nat) return;
-    const GdpDevLayer *Y = uload(&Q->lay) + ((int64_t)ii * max_L + layer);
+    const GdpDevLayer *Y = Q.lay + ((int64_t)ii * max_L + layer);
     const int ntile = uload(&Y->ntile);
     const unsigned nbt = ((unsigned)ntile * ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     const int lo = uload(&Y->lo), hi = uload(&Y->hi);
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     // So all XCDs move up the budget rows of a layer side by side: whatever the band of the layer is,
     // each carries an eighth of it, and what a block waits for -- tiles at and below its own in the
     // layer before -- was handed out a whole layer earlier on every XCD.
-    const unsigned G = (unsigned)uload(&Q->group);
+    const unsigned G = (unsigned)Q.group;
     const unsigned grp = w / G;
     const unsigned bt = (grp * 8u + xcd) * G + (w - grp * G);
     if (bt >= nbt) return;
@@ -444,7 +444,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         const unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
         live = bt >= bt_lo && bt <= bt_hi;   // carries arithmetic; the others only fill or count as done
     }
-    int32_t *cnt_all = uload(&Q->cnt);
+    int32_t *cnt_all = Q.cnt;
     const unsigned q0 = bt * GDP_WAVES_PER_BLOCK;
     if (live && layer >= 1) {
         // the block's first wave waits for everything its four wave tasks read
@@ -455,7 +455,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
             const int d = uload(&Y[-1].dep);
             const int first = t_lo - d < 0 ? 0 : t_lo - d;
             const bool ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, first, t_hi, (int)ntb,
-                                       lane, uload(&Q->abort_flag), uload(&Q->spin_limit));
+                                       lane, Q.abort_flag, Q.spin_limit);
             if (lane == 0) sh_ok = ok ? 1 : 0;
         }
         __syncthreads();
@@ -708,7 +708,7 @@ static hipError_t launch_relax_v(bool marks, const GdpDevLayer *lay, int max_L, 
 
 template <int TS, int R, bool MARKS_BUILT>
 static hipError_t launch_fused_v(bool marks, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
-                          const GdpSched *sched, int layer0)
+                          const GdpSched &sched, int layer0)
 {
     if constexpr (MARKS_BUILT) {
         if (marks) {
@@ -734,7 +734,7 @@ hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int
 #undef X
 }
 
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched *sched, int grid_blocks, int layer0,
+hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
