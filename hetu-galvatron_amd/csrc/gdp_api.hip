@@ -453,19 +453,29 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // the arithmetic of the next; small problems get the shortest (most parallel) one.
         const int ts = pick_ts(g.S, pl->keep_marks);
         const int ntb = (int)align_up((size_t)g.S, (size_t)ts) / ts;
-        // A fused launch takes `chunk` instances at a time through all their layers (in the sorted
-        // order, so mostly instances of one depth): as many as keep two cost buffers each -- the layer
-        // being read and the one being written -- within GALVATRON_DP_CHUNK_MB (default 128) of the
-        // 256 MB memory-side cache.  With all instances of a batch layer by layer instead, a layer's
-        // output has long left that cache when the next layer reads it (256 instances of 24 MB per
-        // layer: 46.9 ms; two at a time: 42.0 ms).
+        // A fused launch can take `chunk` instances at a time through all their layers (in the sorted
+        // order, so mostly instances of one depth) instead of the whole batch layer by layer: as many as
+        // keep two cost buffers each -- the layer being read and the one being written -- within
+        // GALVATRON_DP_CHUNK_MB (default 144) of the 256 MB memory-side cache, so that a layer's output
+        // is still there when the next layer reads it.  Fewer instances in flight also means less work
+        // between a layer and the next, i.e. more waiting; what wins was measured (batches of 96-256
+        // instances, times per solve, layer by layer -> chunked):
+        //   8- and 11-wide tiles, S >= 36: S = 36 14.1 -> 10.8 ms, S = 40 (V = 29493, L = 28) 26.6 -> 21.1,
+        //   S = 44 (V = 65536) 46.8 -> 43.3, S = 56 21.8 -> 16.2, S = 72 25.0 -> 18.1, S = 88 20.5 -> 17.7;
+        //   never slower in 20 shapes; one instance at a time is always slower;
+        //   16-wide tiles (S = 32, 48, 64): 6.4 -> 6.6, 23.2 -> 23.4, 5.7 -> 7.2 -- they issue half the
+        //   cost-row loads per relaxation and do not wait for memory in the first place;
+        //   S = 22..30: 5.0 -> 5.6, 13.4 -> 14.7, 13.9 -> 13.1 -- a block task is over in 2-3 us, and the
+        //   per-task cost of waiting and signalling weighs more than the memory.
+        // So: narrow tiles, at least 36 strategies, and at least two instances that fit.
         {
             size_t pair = 0;  // bytes of two cost buffers of the largest instance
             for (int k = i; k < j; ++k)
                 pair = std::max(pair, 2 * sizeof(double) * ((size_t)g.S + 1) *
                                           ((size_t)inst[(size_t)k].V + (size_t)inst[(size_t)k].P));
-            const size_t budget = env_mb("GALVATRON_DP_CHUNK_MB", 128);
-            g.chunk = (int)std::min<size_t>((size_t)g.count, std::max<size_t>(1, budget / std::max<size_t>(pair, 1)));
+            const size_t fit = env_mb("GALVATRON_DP_CHUNK_MB", 144) / std::max<size_t>(pair, 1);
+            g.chunk = g.count;  // not chunked
+            if (g.S >= 36 && ts <= 11 && fit >= 2 && fit < (size_t)g.count) g.chunk = (int)fit;
             if (pl->chunk_override > 0) g.chunk = std::min(g.count, pl->chunk_override);
         }
         int best_r = 0;
