@@ -169,22 +169,37 @@ struct Group {  // instances with the same S, sorted by L descending
     size_t off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
-// Target-tile width: the one that pads S the least; of two that pad alike the wider one, which
-// issues fewer cost-row loads per relaxation (S = 88: eight blocks of 11 rather than eleven of 8;
-// S = 64: four of 16).  marks: only among the variants built with the argmin table.
-int pick_ts(int S, bool marks)
+// Target-tile width.  With enough work to go round -- `tiles` row tiles of 64 rows in flight together
+// give every wave slot of the device a task -- the width that covers S with the fewest target
+// blocks, of those the one that pads S least, of those the widest (S = 44: three blocks of 15;
+// S = 64: four of 16; S = 36: three of 12).  A problem too small for that is short of parallelism, not
+// of load bandwidth: it takes the next larger block count that fills the device (one instance of S = 44,
+// V = 65536: four blocks of 11, 0.50 ms against 0.67 ms with three of 15), or failing that the most
+// blocks there are.  marks: only among the variants built with the argmin table.
+// GALVATRON_DP_TILE_TS forces a width (tuning aid).
+int pick_ts(int S, bool marks, int64_t tiles, int64_t wave_slots)
 {
-    int best = 0;
-    size_t best_sp = 0;
+    const char *forced = getenv("GALVATRON_DP_TILE_TS");
+    struct Cand { int ts; size_t blocks, sp; };
+    std::vector<Cand> cands;
     for (int v = 0; v < GDP_NUM_VARIANTS; ++v) {
         if (marks && !GDP_VARIANTS[v].marks) continue;
-        const size_t sp = align_up((size_t)S, (size_t)GDP_VARIANTS[v].ts);
-        if (best == 0 || sp < best_sp || (sp == best_sp && GDP_VARIANTS[v].ts > best)) {
-            best = GDP_VARIANTS[v].ts;
-            best_sp = sp;
-        }
+        const int ts = GDP_VARIANTS[v].ts;
+        if (forced && ts == atoi(forced)) return ts;
+        const size_t sp = align_up((size_t)S, (size_t)ts);
+        cands.push_back({ts, sp / (size_t)ts, sp});
     }
-    return best;
+    std::sort(cands.begin(), cands.end(), [](const Cand &a, const Cand &b) {
+        if (a.blocks != b.blocks) return a.blocks < b.blocks;
+        if (a.sp != b.sp) return a.sp < b.sp;
+        return a.ts > b.ts;
+    });
+    for (const Cand &c : cands)
+        if (tiles * (int64_t)c.blocks >= wave_slots) return c.ts;
+    const size_t most = cands.back().blocks;  // not enough work whatever the width: the most tasks
+    for (const Cand &c : cands)
+        if (c.blocks == most) return c.ts;
+    return cands.back().ts;
 }
 
 int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
@@ -451,7 +466,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // Register tile.  Width: least padding of S.  Height: the tallest whose first layer still
         // gives every resident wave at least two tasks, so that the stores of one task drain under
         // the arithmetic of the next; small problems get the shortest (most parallel) one.
-        const int ts = pick_ts(g.S, pl->keep_marks);
+        int64_t tiles64 = 0;
+        for (int k = i; k < j; ++k) tiles64 += ((int64_t)inst[(size_t)k].V + 63) / 64;
+        const int ts = pick_ts(g.S, pl->keep_marks, tiles64, wave_slots);
         const int ntb = (int)align_up((size_t)g.S, (size_t)ts) / ts;
         // A fused launch can take `chunk` instances at a time through all their layers (in the sorted
         // order, so mostly instances of one depth) instead of the whole batch layer by layer: as many as
@@ -467,7 +484,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         //   cost-row loads per relaxation and do not wait for memory in the first place;
         //   S = 22..30: 5.0 -> 5.6, 13.4 -> 14.7, 13.9 -> 13.1 -- a block task is over in 2-3 us, and the
         //   per-task cost of waiting and signalling weighs more than the memory.
-        // So: narrow tiles, at least 36 strategies, and at least two instances that fit.
+        // So: narrow tiles, at least 36 strategies, and at least two instances that fit.  (With the widths
+        // 12 to 16 picked for S >= 36 by now, this happens only where a narrow tile is forced; with those
+        // widths chunking changed the same batches by -9 % to +9 %, so it is left to GALVATRON_DP_CHUNK.)
         {
             size_t pair = 0;  // bytes of two cost buffers of the largest instance
             for (int k = i; k < j; ++k)
@@ -475,7 +494,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                                           ((size_t)inst[(size_t)k].V + (size_t)inst[(size_t)k].P));
             const size_t fit = env_mb("GALVATRON_DP_CHUNK_MB", 144) / std::max<size_t>(pair, 1);
             g.chunk = g.count;  // not chunked
-            if (g.S >= 36 && ts <= 11 && fit >= 2 && fit < (size_t)g.count) g.chunk = (int)fit;
+            if (g.S >= 36 && ts <= 11 && !pl->keep_marks && fit >= 2 && fit < (size_t)g.count) g.chunk = (int)fit;
             if (pl->chunk_override > 0) g.chunk = std::min(g.count, pl->chunk_override);
         }
         int best_r = 0;

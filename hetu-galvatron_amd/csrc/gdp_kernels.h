@@ -109,16 +109,24 @@ struct GdpDevOut {
 };
 
 // Register tile of the relaxation kernel: TS target strategies x (64 lanes x R rows) per wavefront.
-// Variants of one width are listed tallest first.  A wider tile issues fewer cost-row loads per
-// relaxation (one 512-byte load feeds 2*TS vector instructions); the 16-wide ones exist for the
-// costs-only relaxation alone: with the argmin tracked as well they would not fit the registers.
+// Variants of one width are listed tallest first.  The host picks the width that covers S with the
+// fewest target blocks: every block of a row tile reads all of the tile's source rows again, and a
+// wave task's time is set by that stream of loads rather than by its arithmetic (measured on batches
+// of 96-256 instances, ms per solve by width: S = 44: 8 -> 30.4, 11 -> 24.5, 15 -> 20.3; S = 40:
+// 8 -> 27.8, 15 -> 18.9; S = 88: 11 -> 20.6, 15 -> 17.4; S = 56: 8 -> 22.0, 14 -> 15.6), then the one
+// that pads S least.  Widths 12 to 16 exist for the costs-only relaxation alone: with the argmin
+// tracked as well they would not fit the registers (the transition costs of a step alone take
+// 4*TS scalar registers, double-buffered).
 struct GdpVariant {
     int ts, r;
     bool marks;  // also built with the argmin table
 };
-static const GdpVariant GDP_VARIANTS[] = {{16, 3, false}, {16, 2, false}, {16, 1, false}, {8, 4, true}, {8, 2, true},
-                                          {8, 1, true},   {11, 3, true},  {11, 2, true},  {11, 1, true}};
-#define GDP_NUM_VARIANTS 9
+static const GdpVariant GDP_VARIANTS[] = {
+    {16, 3, false}, {16, 2, false}, {16, 1, false}, {15, 3, false}, {15, 2, false}, {15, 1, false},
+    {14, 3, false}, {14, 2, false}, {14, 1, false}, {13, 3, false}, {13, 2, false}, {13, 1, false},
+    {12, 3, false}, {12, 2, false}, {12, 1, false}, {11, 3, true},  {11, 2, true},  {11, 1, true},
+    {8, 4, true},   {8, 2, true},   {8, 1, true}};
+#define GDP_NUM_VARIANTS 21
 
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
 // marks: track and store the argmin table (otherwise costs only).  lay: the group's table of

@@ -690,9 +690,12 @@ static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, 
 }
 
 // one entry per element of GDP_VARIANTS, in the same order: (index, TS, R, built with the argmin table)
-#define GDP_FOR_EACH_VARIANT(X)                                                                          \
-    X(0, 16, 3, false) X(1, 16, 2, false) X(2, 16, 1, false) X(3, 8, 4, true) X(4, 8, 2, true) X(5, 8, 1, true) \
-    X(6, 11, 3, true) X(7, 11, 2, true) X(8, 11, 1, true)
+#define GDP_FOR_EACH_VARIANT(X)                                                                       \
+    X(0, 16, 3, false) X(1, 16, 2, false) X(2, 16, 1, false) X(3, 15, 3, false) X(4, 15, 2, false)        \
+    X(5, 15, 1, false) X(6, 14, 3, false) X(7, 14, 2, false) X(8, 14, 1, false) X(9, 13, 3, false)        \
+    X(10, 13, 2, false) X(11, 13, 1, false) X(12, 12, 3, false) X(13, 12, 2, false) X(14, 12, 1, false)   \
+    X(15, 11, 3, true) X(16, 11, 2, true) X(17, 11, 1, true) X(18, 8, 4, true) X(19, 8, 2, true)          \
+    X(20, 8, 1, true)
 
 template <int TS, int R, bool MARKS_BUILT>
 static hipError_t launch_relax_v(bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile, int SP, int layer,

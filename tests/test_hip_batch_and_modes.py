@@ -153,9 +153,10 @@ def test_instances_taken_through_the_launch_a_few_at_a_time(golden, monkeypatch,
             plan.fetch()
             for n, prob in zip(names, probs):
                 _check_against_golden(prob, golden[n], f"{n} chunk={chunk} rows={max_rows}")
-    assert t.fused
-    if max_rows < 10:
-        assert t.relax_launches > 4
+    if "GALVATRON_DP_FUSED" not in os.environ:          # a preset in the environment overrides the flag
+        assert t.fused
+        if max_rows < 10:
+            assert t.relax_launches > 4
 
 
 def test_device_memory_short_for_one_buffer_per_layer(golden, monkeypatch):

@@ -18,7 +18,8 @@ SHAPES = [(1, 1, 1), (1, 1, 7), (2, 1, 64), (3, 2, 65), (4, 7, 191), (3, 8, 192)
           (6, 11, 256), (3, 12, 257), (4, 16, 383), (2, 21, 385), (7, 22, 512), (3, 23, 700), (2, 33, 129),
           (3, 44, 1000), (2, 45, 130), (2, 63, 300), (3, 64, 333), (2, 65, 200), (2, 88, 410), (1, 127, 150),
           (2, 128, 140), (2, 129, 131), (1, 255, 90), (2, 256, 70), (9, 5, 2048), (12, 3, 4099), (20, 4, 1500),
-          (2, 257, 70), (2, 300, 150), (1, 513, 40)]
+          (2, 257, 70), (2, 300, 150), (1, 513, 40), (3, 13, 200), (3, 14, 333), (2, 26, 300), (2, 28, 129),
+          (2, 39, 150), (2, 42, 200), (2, 52, 140), (2, 56, 190), (2, 60, 130), (2, 74, 100)]
 
 
 def _compare(inst, tag, launch=None):
