@@ -175,7 +175,7 @@ struct Group {  // instances with the same S, sorted by L descending
 // S = 64: four of 16; S = 36: three of 12).  A problem too small for that is short of parallelism, not
 // of load bandwidth: it takes the next larger block count that fills the device (one instance of S = 44,
 // V = 65536: four blocks of 11, 0.50 ms against 0.67 ms with three of 15), or failing that the most
-// blocks there are.  marks: only among the variants built with the argmin table.
+// blocks there are.  marks: only among the variants built with the argmin table, by least padding.
 // GALVATRON_DP_TILE_TS forces a width (tuning aid).
 int pick_ts(int S, bool marks, int64_t tiles, int64_t wave_slots)
 {
@@ -188,6 +188,14 @@ int pick_ts(int S, bool marks, int64_t tiles, int64_t wave_slots)
         if (forced && ts == atoi(forced)) return ts;
         const size_t sp = align_up((size_t)S, (size_t)ts);
         cands.push_back({ts, sp / (size_t)ts, sp});
+    }
+    if (marks) {
+        // five vector instructions per relaxation: the arithmetic binds, so the least padding decides
+        // (S = 64: eight blocks of 8, 5.9 ms; six of 11, padded to 66, 6.3 ms)
+        const Cand *best = &cands[0];
+        for (const Cand &c : cands)
+            if (c.sp < best->sp || (c.sp == best->sp && c.ts > best->ts)) best = &c;
+        return best->ts;
     }
     std::sort(cands.begin(), cands.end(), [](const Cand &a, const Cand &b) {
         if (a.blocks != b.blocks) return a.blocks < b.blocks;
