@@ -613,7 +613,48 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
         const double *inter = uload(&I->inter);
         const double *intra = uload(&I->intra);
         const int32_t *inter_index = uload(&I->inter_index);
-        for (int i = L - 1; i > 0; --i) {
+        int i = L - 1;
+        if (S <= 64) {
+            // Up to 64 strategies: lane s keeps what layer i holds for strategy s -- memory cost, row
+            // offset, intra cost -- fetched one layer ahead, so that the step from a cell to its
+            // predecessor is a lane read, one round of gathered loads (cost row and transition column
+            // together) and the reduction, instead of a dependent scalar load before the gather.
+            const int sl = lane < S ? lane : S - 1;
+            int m_next = mem[(int64_t)i * S + sl];
+            int64_t r_next = roff[(int64_t)i * rows + sl];
+            double a_next = intra[(int64_t)i * SP + sl];
+            int t_next = uload(inter_index + i);
+            for (; i > 0; --i) {
+                const int cur = idx;
+                const int m_cur = m_next;
+                const int64_t r_cur = r_next;
+                const double a_cur = a_next;
+                const int t_cur = t_next;
+                if (i > 1) {
+                    m_next = mem[(int64_t)(i - 1) * S + sl];
+                    r_next = roff[(int64_t)(i - 1) * rows + sl];
+                    a_next = intra[(int64_t)(i - 1) * SP + sl];
+                    t_next = uload(inter_index + (i - 1));
+                }
+                v -= __builtin_amdgcn_readlane(m_cur, cur);  // the source row of cell (i, v, cur)
+                if (v < 0) break;
+                const double *src = H + (int64_t)(i % nbuf) * hstride;  // costs before layer i
+                const double a = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(a_cur), cur),
+                                                  __builtin_amdgcn_readlane(__double2loint(a_cur), cur));
+                double bv = INFINITY;
+                int bi = 0x7fffffff;
+                if (lane < S) {
+                    bv = (src[r_cur + v] + inter[((int64_t)t_cur * rows + lane) * SP + cur]) + a;
+                    bi = lane;
+                }
+                wave_argmin(bv, bi);
+                idx = __builtin_amdgcn_readfirstlane(bi);
+                if (idx >= S) { v = -1; break; }
+                if (lane == 0) path[i - 1] = idx;
+            }
+            i = 0;
+        }
+        for (; i > 0; --i) {
             const int cur = idx;
             v -= uload(mem + (int64_t)i * S + cur);  // the source row of cell (i, v, cur)
             if (v < 0) break;
