@@ -445,6 +445,19 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         live = bt >= bt_lo && bt <= bt_hi;   // carries arithmetic; the others only fill or count as done
     }
     int32_t *cnt_all = Q.cnt;
+    // touch what the task reads first (row offsets, first transition costs), so that it sits in the
+    // scalar cache by the time the wait is over
+    int64_t pf_o = 0;
+    double pf_a = 0, pf_b = 0;
+    if (live) {
+        const unsigned qq = bt * GDP_WAVES_PER_BLOCK + wave;
+        const unsigned tl = qq / ntb, tbb = qq - tl * ntb;
+        const int64_t *ro_ = uload(&Y->ro);
+        const double *it_ = uload(&Y->it) + tbb * TS;
+        pf_o = uload(ro_);
+        pf_a = uload(it_);
+        pf_b = uload(it_ + (TS - 1));
+    }
     const unsigned q0 = bt * GDP_WAVES_PER_BLOCK;
     if (live && layer >= 1) {
         // the block's first wave waits for everything its four wave tasks read
@@ -461,6 +474,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         __syncthreads();
         if (__builtin_amdgcn_readfirstlane(sh_ok) == 0) return;  // the launch is being abandoned
     }
+    asm volatile("" ::"s"(pf_o), "s"(pf_a), "s"(pf_b));
     const unsigned q = q0 + wave;
     const unsigned tile = q / ntb;
     const unsigned tb = q - tile * ntb;
