@@ -170,6 +170,7 @@ def main() -> int:
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
             "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
+            "tile": "%d target strategies x %d budget rows per wavefront" % (tm.tile_ts, 64 * tm.tile_r),
             "kernel": "gdp_relax_fused_kernel" if tm.fused else "gdp_relax_kernel",
         }
 
@@ -184,6 +185,7 @@ def main() -> int:
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
                    "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
+                   "register_tile": m["tile"],
                    "relaxations_executed_fraction": m["executed_fraction"], "device": _lib.device_info()},
         "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
                      "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,

@@ -901,6 +901,13 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
         t->relax_bytes = pl->relax_bytes;
         t->relax_launches = (int32_t)launches;
         t->fused = pl->fused ? 1 : 0;
+        if (!pl->groups.empty()) {
+            const Group &g0 = pl->groups.front();
+            t->tile_ts = GDP_VARIANTS[g0.variant].ts;
+            t->tile_r = GDP_VARIANTS[g0.variant].r;
+            t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
+        }
+        t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));
         if (mode >= 2) {
             float sum = 0;

@@ -98,6 +98,11 @@ typedef struct gdp_timing {
     double executed;       /* relaxations actually carried out: cells whose sources are all +inf, and cells
                               that no requested start row can reach back to, are not computed           */
     double relax_bytes;    /* algorithmic HBM bytes of the relaxation kernels (f read+write, argmin write if kept) */
+    /* how the plan was laid out (of its first group of instances with one S) */
+    int32_t tile_ts;       /* target strategies per register tile                               */
+    int32_t tile_r;        /* budget rows per lane                                              */
+    int32_t keep_marks;    /* 1: the argmin table is stored while relaxing                      */
+    int32_t chunk;         /* instances taken through a fused launch together; 0: all, layer by layer */
 } gdp_timing;
 
 typedef struct gdp_plan gdp_plan;

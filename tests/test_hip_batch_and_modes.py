@@ -159,6 +159,27 @@ def test_instances_taken_through_the_launch_a_few_at_a_time(golden, monkeypatch,
             assert t.relax_launches > 4
 
 
+def test_plan_reports_its_layout(golden):
+    """The register tile follows the documented rule: fewest target blocks that still fill the device
+    (costs only), least padding with the argmin table; the timing record says what was chosen."""
+    if any(k in os.environ for k in ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R")):
+        pytest.skip("the environment presets the layout")
+
+    def layout(insts, **kw):
+        with _lib.Plan([_problem(i, **kw) for i in insts]) as plan:
+            t = plan.run(1)
+        return t.tile_ts, t.keep_marks
+
+    small64 = H.build_case(golden["cfg2_small"])                # one instance, S = 64, V = 12288: under-filled
+    assert layout([small64]) == (8, 0)                          # the most blocks there are
+    assert layout([small64] * 24) == (16, 0)                    # enough work: four blocks of 16
+    assert layout([small64] * 24, keep_marks=True) == (8, 1)    # argmin table: least padding among 8 / 11
+    s44 = [H.build_case(golden["cfg3_smallV_%d" % i]) for i in range(8)]   # S = 44, V = 8192
+    assert layout(s44 * 8) == (15, 0)                           # three blocks of 15
+    assert layout(s44 * 8, keep_marks=True) == (11, 1)
+    assert layout([H.build_case(golden["cfg4_small"])] * 16)[0] == 15      # S = 88: six blocks of 15
+
+
 def test_device_memory_short_for_one_buffer_per_layer(golden, monkeypatch):
     """A device too full for one cost buffer per layer: plan creation starts over with two cost
     buffers and the argmin table (and the register tiles that exist for that mode; S = 64 uses a
