@@ -1,6 +1,6 @@
 """Differential test on the GPU: seeded random instances through the plugin signature against
 the C oracle, on shapes chosen to hit the kernel's corners: S around the register-tile widths
-(8, 11) and the wavefront width (63..65, 127..129, 255..257, 300, 513), V not a multiple of any tile height,
+(8, 11) and the wavefront width (63..65, 127..129, 255..257, 300, 513, 1000, 1024 = the largest), V not a multiple of any tile height,
 memory costs near 1, near V and above V, +inf costs, exact ties, shared and per-layer inter
 matrices, start rows below 0.  Full f and mark arrays are compared as well as the results."""
 import os
@@ -19,7 +19,8 @@ SHAPES = [(1, 1, 1), (1, 1, 7), (2, 1, 64), (3, 2, 65), (4, 7, 191), (3, 8, 192)
           (3, 44, 1000), (2, 45, 130), (2, 63, 300), (3, 64, 333), (2, 65, 200), (2, 88, 410), (1, 127, 150),
           (2, 128, 140), (2, 129, 131), (1, 255, 90), (2, 256, 70), (9, 5, 2048), (12, 3, 4099), (20, 4, 1500),
           (2, 257, 70), (2, 300, 150), (1, 513, 40), (3, 13, 200), (3, 14, 333), (2, 26, 300), (2, 28, 129),
-          (2, 39, 150), (2, 42, 200), (2, 52, 140), (2, 56, 190), (2, 60, 130), (2, 74, 100)]
+          (2, 39, 150), (2, 42, 200), (2, 52, 140), (2, 56, 190), (2, 60, 130), (2, 74, 100), (1, 1000, 33),
+          (1, 1024, 30)]
 
 
 def _compare(inst, tag, launch=None):
