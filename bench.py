@@ -117,7 +117,7 @@ def main() -> int:
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs the DP hot path on ONE GPU; --gpus must be 1 "
-              "(instances of a batch are independent and would shard by instance, see DESIGN.md)", file=sys.stderr)
+              "(instances of a batch are independent and would shard by instance with no exchange)", file=sys.stderr)
         return 2
 
     import ctypes

@@ -26,7 +26,7 @@ def _check_against_golden(prob, rec, name):
 
 
 def test_batched_sweep_256_instances_matches_reference(golden):
-    """BASELINE config 3: all 256 instances of the pp x bsz x chunks sweep in ONE gdp_solve_batch
+    """Workload cfg3: all 256 instances of the pp x bsz x chunks sweep in ONE gdp_solve_batch
     call, every instance compared with the reference's result for it."""
     insts = W.config3()
     assert len(insts) == 256
