@@ -141,6 +141,96 @@ void arena_give(int device, char *ptr, size_t bytes)
     for (const Arena &a : drop) (void)hipFree(a.ptr);  // same device as the caller's plan
 }
 
+// ---- streams kept between plans --------------------------------------------------------------------
+// Creating and destroying a stream costs more than solving a small DP (0.14 ms against 0.4 ms), and
+// a search makes thousands of such calls in a row.  A finished plan therefore hands its stream, its
+// two events and its page-locked read-back buffer to the next plan on that device; at most
+// LANES_KEPT wait here, gdp_cache_trim() releases them.
+struct Lane {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    char *back = nullptr;  // page-locked host memory the results are copied into
+    size_t back_bytes = 0;
+};
+constexpr size_t LANES_KEPT = 64;
+std::mutex g_lane_mu;
+std::vector<Lane> g_lanes;
+
+void lane_release(Lane &ln)  // the lane's device is current
+{
+    if (ln.ev_begin) (void)hipEventDestroy(ln.ev_begin);
+    if (ln.ev_end) (void)hipEventDestroy(ln.ev_end);
+    if (ln.stream) (void)hipStreamDestroy(ln.stream);
+    if (ln.back) (void)hipHostFree(ln.back);
+    ln = Lane();
+}
+
+hipError_t lane_take(int device, size_t back_bytes, Lane *out)
+{
+    Lane ln;
+    {
+        std::lock_guard<std::mutex> lk(g_lane_mu);
+        for (size_t i = g_lanes.size(); i-- > 0;)
+            if (g_lanes[i].device == device) {
+                ln = g_lanes[i];
+                g_lanes.erase(g_lanes.begin() + (long)i);
+                break;
+            }
+    }
+    hipError_t e = hipSuccess;
+    if (!ln.stream) {
+        ln.device = device;
+        e = hipStreamCreateWithFlags(&ln.stream, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipEventCreate(&ln.ev_begin);
+        if (e == hipSuccess) e = hipEventCreate(&ln.ev_end);
+    }
+    if (e == hipSuccess && ln.back_bytes < back_bytes) {
+        if (ln.back) (void)hipHostFree(ln.back);
+        ln.back = nullptr;
+        ln.back_bytes = 0;
+        const size_t want = align_up(back_bytes, 65536);
+        e = hipHostMalloc((void **)&ln.back, want, hipHostMallocDefault);
+        if (e == hipSuccess) ln.back_bytes = want;
+    }
+    if (e != hipSuccess) {
+        lane_release(ln);
+        return e;
+    }
+    *out = ln;
+    return hipSuccess;
+}
+
+void lane_give(Lane &ln)  // the lane's device is current and its stream idle
+{
+    if (!ln.stream) return;
+    {
+        std::lock_guard<std::mutex> lk(g_lane_mu);
+        if (g_lanes.size() < LANES_KEPT && ln.back_bytes <= ((size_t)64 << 20)) {
+            g_lanes.push_back(ln);
+            ln = Lane();
+            return;
+        }
+    }
+    lane_release(ln);
+}
+
+void lane_trim()
+{
+    std::vector<Lane> drop;
+    {
+        std::lock_guard<std::mutex> lk(g_lane_mu);
+        drop.swap(g_lanes);
+    }
+    int cur = 0;
+    (void)hipGetDevice(&cur);
+    for (Lane &ln : drop) {
+        (void)hipSetDevice(ln.device);
+        lane_release(ln);
+    }
+    (void)hipSetDevice(cur);
+}
+
 struct HostInst {
     int orig;  // index in the caller's arrays
     int L, V, S, SP, SU, P, ntile, n_key, n_inter, variant, nbuf;
@@ -233,11 +323,16 @@ struct gdp_plan {
     int n_key_total = 0;
     size_t n_res_total = 0;
     int max_L = 0;
-    hipStream_t stream = nullptr;
+    Lane lane;                   // stream, events and read-back buffer, taken from / returned to the pool
+    hipStream_t stream = nullptr;    // = lane.stream
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     std::vector<hipEvent_t> ev_relax;  // pairs
-    std::vector<GdpDevOut> h_out;
-    std::vector<int32_t> h_res;
+    // What a run copies back in one piece: abort flag, per-key outputs, strategy lists (device offsets
+    // off_abort .. off_res + its size; the same offsets relative to off_abort inside lane.back).
+    size_t back_bytes = 0;
+    const GdpDevOut *h_out = nullptr;
+    const int32_t *h_res = nullptr;
+    std::vector<char> stage;     // host copy of the inputs' device layout; the upload reads it asynchronously
     double relaxations = 0, relax_bytes = 0;
     double executed = 0;     // relaxations actually carried out (tiles inside the bands)
     bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
@@ -324,15 +419,11 @@ int validate(const gdp_problem *p, int i)
 void destroy(gdp_plan *pl)
 {
     if (!pl) return;
-    if (pl->dbase) {
-        (void)hipSetDevice(pl->device);
-        if (pl->stream) (void)hipStreamSynchronize(pl->stream);
-        arena_give(pl->device, pl->dbase, pl->dalloc);
-    }
+    if (pl->dbase || pl->lane.stream) (void)hipSetDevice(pl->device);
+    if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read pl->stage
+    if (pl->dbase) arena_give(pl->device, pl->dbase, pl->dalloc);
     for (hipEvent_t e : pl->ev_relax) (void)hipEventDestroy(e);
-    if (pl->ev_begin) (void)hipEventDestroy(pl->ev_begin);
-    if (pl->ev_end) (void)hipEventDestroy(pl->ev_end);
-    if (pl->stream) (void)hipStreamDestroy(pl->stream);
+    lane_give(pl->lane);
     delete pl;
 }
 
@@ -608,15 +699,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
     }
     const size_t small_bytes = off;
-    // words that every run resets to zero: abort flag, ticket counters, completion counters
+    // words that every fused run resets to zero: completion counters, abort flag
     pl->off_zero = off;
-    pl->off_abort = take(sizeof(int32_t));
     for (auto &g : pl->groups) {
         g.off_cnt = take(sizeof(int32_t) * (size_t)g.count * g.max_L * g.max_ntile);
     }
+    pl->off_abort = take(sizeof(int32_t));
     pl->zero_words = (off - pl->off_zero) / sizeof(int32_t);
+    // abort flag, per-key outputs and strategy lists lie together: a run copies them back in one piece
     pl->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(nk, 1));
     pl->off_res = take(sizeof(int32_t) * std::max<size_t>(nres, 1));
+    pl->back_bytes = off - pl->off_abort;
     const size_t fixed_bytes = off;
     // One cost buffer per layer lets all layers share a launch and lets the backtrack recompute the
     // argmin of the cells it visits, so that the relaxation does not have to track it.  If that does
@@ -652,7 +745,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         return fail_hip(e, buf);
     }
     // ---- build the small region on the host ------------------------------------------------------
-    std::vector<char> stage;
+    std::vector<char> &stage = pl->stage;
     try {
         stage.assign(small_bytes, 0);
     } catch (const std::bad_alloc &) {
@@ -812,9 +905,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
-    GDP_HIP(hipStreamCreateWithFlags(&pl->stream, hipStreamNonBlocking));
-    GDP_HIP(hipEventCreate(&pl->ev_begin));
-    GDP_HIP(hipEventCreate(&pl->ev_end));
+    {
+        const hipError_t e = lane_take(pl->device, pl->back_bytes, &pl->lane);
+        if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
+            (void)hipGetLastError();
+            return fail(GDP_E_NOMEM, "page-locked host memory for the results");
+        }
+        GDP_HIP(e);
+        pl->stream = pl->lane.stream;
+        pl->ev_begin = pl->lane.ev_begin;
+        pl->ev_end = pl->lane.ev_end;
+    }
     GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
@@ -822,10 +923,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, GDP_INIT_PADS | GDP_INIT_ZERO,
                                     pl->stream));
     }
-    GDP_HIP(hipStreamSynchronize(pl->stream));
+    // no wait here: the stream orders the upload and these fills before the first run, pl->stage stays
+    // alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);
-    pl->h_out.resize((size_t)std::max(nk, 1));
-    pl->h_res.resize(std::max<size_t>(nres, 1));
     return GDP_OK;
 }
 
@@ -879,10 +979,13 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     }
     GDP_HIP(gdp_launch_epilogue(pl->keep_marks, d_insts, d_keys, pl->n_key_total, d_out, d_res, pl->stream));
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
-    int32_t aborted = 0;
-    if (pl->fused)
-        GDP_HIP(hipMemcpyAsync(&aborted, pl->dbase + pl->off_abort, sizeof aborted, hipMemcpyDeviceToHost, pl->stream));
+    GDP_HIP(hipMemcpyAsync(pl->lane.back, pl->dbase + pl->off_abort, pl->back_bytes, hipMemcpyDeviceToHost,
+                           pl->stream));
     GDP_HIP(hipStreamSynchronize(pl->stream));
+    pl->h_out = reinterpret_cast<const GdpDevOut *>(pl->lane.back + (pl->off_out - pl->off_abort));
+    pl->h_res = reinterpret_cast<const int32_t *>(pl->lane.back + (pl->off_res - pl->off_abort));
+    // the flag is cleared and written by fused launches only
+    const int32_t aborted = pl->fused ? *reinterpret_cast<const int32_t *>(pl->lane.back) : 0;
     if (aborted) {
         // Not every block of the fused launch was resident (the device is shared) or a wait ran out:
         // nothing of that run is kept; do the same work with one launch per layer instead.
@@ -926,13 +1029,7 @@ int fetch(gdp_plan *pl, gdp_result *const *r)
 {
     if (!pl->ran) return fail(GDP_E_BADARG, "gdp_plan_fetch before gdp_plan_run");
     GDP_HIP(hipSetDevice(pl->device));
-    if (pl->n_key_total > 0) {
-        GDP_HIP(hipMemcpyAsync(pl->h_out.data(), pl->dbase + pl->off_out, sizeof(GdpDevOut) * (size_t)pl->n_key_total,
-                               hipMemcpyDeviceToHost, pl->stream));
-        GDP_HIP(hipMemcpyAsync(pl->h_res.data(), pl->dbase + pl->off_res, sizeof(int32_t) * pl->n_res_total,
-                               hipMemcpyDeviceToHost, pl->stream));
-        GDP_HIP(hipStreamSynchronize(pl->stream));
-    }
+    // the run has already copied the outputs into the plan's page-locked buffer
     const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
     for (int i = 0; i < pl->n; ++i) {
         const HostInst &h = pl->inst[(size_t)i];
@@ -944,7 +1041,7 @@ int fetch(gdp_plan *pl, gdp_result *const *r)
             out->total[k] = o.total;
             out->remaining[k] = o.remaining;
             if (o.feasible)
-                memcpy(out->res + (size_t)k * h.L, pl->h_res.data() + h.res_begin + (size_t)k * h.L,
+                memcpy(out->res + (size_t)k * h.L, pl->h_res + h.res_begin + (size_t)k * h.L,
                        sizeof(int32_t) * (size_t)h.L);
         }
         if ((h.flags & GDP_EXPORT_F) && out->f_out) {
@@ -1054,7 +1151,11 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
 
 void gdp_plan_destroy(gdp_plan *plan) { destroy(plan); }
 
-void gdp_cache_trim(void) { arena_trim(-1); }
+void gdp_cache_trim(void)
+{
+    arena_trim(-1);
+    lane_trim();
+}
 
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
 {

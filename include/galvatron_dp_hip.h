@@ -147,7 +147,9 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
 
 /* Frees the device allocations that finished plans left behind for reuse (no counterpart in the
  * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 16384, 0 keeps
- * nothing), because obtaining device memory costs far more than a solve. */
+ * nothing), because obtaining device memory costs far more than a solve.  Finished plans also leave
+ * their stream, two events and page-locked result buffer for the next plan (at most 64 sets; creating
+ * and destroying a stream takes a third as long as a small solve); this call releases those too. */
 void gdp_cache_trim(void);
 
 /* Text of the calling thread's last error ("" if none). */

@@ -135,6 +135,32 @@ def test_batch_solved_in_parts_and_allocation_reuse(golden, monkeypatch):
         _check_against_golden(prob, golden[n], n)
 
 
+def test_streams_and_result_buffers_handed_from_plan_to_plan(golden):
+    """A finished plan leaves its stream and page-locked result buffer to the next plan.  Plans whose
+    results are smaller, then larger than the buffer they inherit, plans alive at the same time (each
+    needs a set of its own), fetch after a later plan has run, and giving everything back in between."""
+    small = ["ties_2", "infeasible_2", "rand_2"]
+    big = ["cfg3_smallV_%d" % i for i in range(8)] * 40          # 320 instances: > 64 KB of results
+    for rep in range(3):
+        for names in (small, big, small[:1]):
+            probs = [_problem(H.build_case(golden[n])) for n in names]
+            _lib.solve_batch(probs)
+            for n, prob in zip(names, probs):
+                _check_against_golden(prob, golden[n], f"{n} rep {rep}")
+        if rep == 1:
+            _lib.cache_trim()
+    pa = [_problem(H.build_case(golden[n])) for n in small]
+    pb = [_problem(H.build_case(golden[n])) for n in big[:8]]
+    with _lib.Plan(pa) as a, _lib.Plan(pb) as b:
+        a.run()
+        b.run()
+        b.run()
+        a.fetch()               # a's results were copied back by a's own run, into a's own buffer
+        b.fetch()
+    for n, prob in zip(small + big[:8], pa + pb):
+        _check_against_golden(prob, golden[n], n)
+
+
 @pytest.mark.parametrize("chunk,max_rows", [(1, 65535), (3, 65535), (2, 5), (1000, 3), (4, 1)])
 def test_instances_taken_through_the_launch_a_few_at_a_time(golden, monkeypatch, chunk, max_rows):
     """A fused launch takes `chunk` instances at a time through all their layers (grid rows follow a
