@@ -45,8 +45,10 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Getting fresh device memory costs far more than filling it (94 GB for 256 Llama-7B-like instances:
 // 2.7 s to allocate, 0.05 s to solve), and the search engine solves thousands of DPs in a row.  The
 // allocation of a finished plan is therefore kept for the next plan on that device instead of being
-// freed: up to GALVATRON_DP_CACHE_MB (default 16384, 0 = keep nothing) in total, the largest kept
-// ones given up first when that is exceeded, all of them on an out-of-memory error or gdp_cache_trim().
+// freed: up to GALVATRON_DP_CACHE_MB (default 20480, 0 = keep nothing) in total -- room for the two
+// allocations of GALVATRON_DP_ARENA_MB that a batch solved in parts works in, and the small ones of
+// single solves between such batches --, the ones given back longest ago given up first when that is
+// exceeded, all of them on an out-of-memory error or gdp_cache_trim().
 struct Arena {
     int device;
     char *ptr;
@@ -120,7 +122,7 @@ hipError_t arena_take(int device, size_t need, char **ptr, size_t *bytes)
 
 void arena_give(int device, char *ptr, size_t bytes)
 {
-    const size_t cap = env_mb("GALVATRON_DP_CACHE_MB", 16384);
+    const size_t cap = env_mb("GALVATRON_DP_CACHE_MB", 20480);
     std::vector<Arena> drop;
     if (bytes > cap) {
         drop.push_back({device, ptr, bytes});
@@ -129,13 +131,10 @@ void arena_give(int device, char *ptr, size_t bytes)
         g_arenas.push_back({device, ptr, bytes});
         size_t total = 0;
         for (const Arena &a : g_arenas) total += a.bytes;
-        while (total > cap) {  // the largest first: small ones serve the many small solves
-            size_t big = 0;
-            for (size_t i = 1; i < g_arenas.size(); ++i)
-                if (g_arenas[i].bytes > g_arenas[big].bytes) big = i;
-            total -= g_arenas[big].bytes;
-            drop.push_back(g_arenas[big]);
-            g_arenas.erase(g_arenas.begin() + (long)big);
+        while (total > cap) {  // the one given back longest ago first (they are kept in that order)
+            total -= g_arenas.front().bytes;
+            drop.push_back(g_arenas.front());
+            g_arenas.erase(g_arenas.begin());
         }
     }
     for (const Arena &a : drop) (void)hipFree(a.ptr);  // same device as the caller's plan
@@ -152,6 +151,8 @@ struct Lane {
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     char *back = nullptr;  // page-locked host memory the results are copied into
     size_t back_bytes = 0;
+    char *up = nullptr;    // page-locked host memory the inputs' device layout is built in (may be absent)
+    size_t up_bytes = 0;
 };
 constexpr size_t LANES_KEPT = 64;
 std::mutex g_lane_mu;
@@ -163,10 +164,29 @@ void lane_release(Lane &ln)  // the lane's device is current
     if (ln.ev_end) (void)hipEventDestroy(ln.ev_end);
     if (ln.stream) (void)hipStreamDestroy(ln.stream);
     if (ln.back) (void)hipHostFree(ln.back);
+    if (ln.up) (void)hipHostFree(ln.up);
     ln = Lane();
 }
 
-hipError_t lane_take(int device, size_t back_bytes, Lane *out)
+// Page-locked memory of at least `bytes` behind *ptr (grown in steps of `grain`, contents not kept).
+hipError_t pinned_reserve(char **ptr, size_t *have, size_t bytes, size_t grain)
+{
+    if (*have >= bytes) return hipSuccess;
+    if (*ptr) (void)hipHostFree(*ptr);
+    *ptr = nullptr;
+    *have = 0;
+    const size_t want = align_up(bytes, grain);
+    const hipError_t e = hipHostMalloc((void **)ptr, want, hipHostMallocDefault);
+    if (e == hipSuccess) *have = want;
+    return e;
+}
+
+// Inputs up to this size are laid out in page-locked memory: the upload then is one asynchronous DMA
+// (a 0.4 MB upload from pageable memory holds the calling thread for 0.17 ms).  Larger ones are
+// built in ordinary memory; their upload is a small part of their solve.
+constexpr size_t UPLOAD_PINNED_MAX = (size_t)16 << 20;
+
+hipError_t lane_take(int device, size_t back_bytes, size_t up_bytes, Lane *out)
 {
     Lane ln;
     {
@@ -185,14 +205,8 @@ hipError_t lane_take(int device, size_t back_bytes, Lane *out)
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_begin);
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_end);
     }
-    if (e == hipSuccess && ln.back_bytes < back_bytes) {
-        if (ln.back) (void)hipHostFree(ln.back);
-        ln.back = nullptr;
-        ln.back_bytes = 0;
-        const size_t want = align_up(back_bytes, 65536);
-        e = hipHostMalloc((void **)&ln.back, want, hipHostMallocDefault);
-        if (e == hipSuccess) ln.back_bytes = want;
-    }
+    if (e == hipSuccess) e = pinned_reserve(&ln.back, &ln.back_bytes, back_bytes, 65536);
+    if (e == hipSuccess && up_bytes <= UPLOAD_PINNED_MAX) e = pinned_reserve(&ln.up, &ln.up_bytes, up_bytes, (size_t)1 << 20);
     if (e != hipSuccess) {
         lane_release(ln);
         return e;
@@ -206,7 +220,7 @@ void lane_give(Lane &ln)  // the lane's device is current and its stream idle
     if (!ln.stream) return;
     {
         std::lock_guard<std::mutex> lk(g_lane_mu);
-        if (g_lanes.size() < LANES_KEPT && ln.back_bytes <= ((size_t)64 << 20)) {
+        if (g_lanes.size() < LANES_KEPT && ln.back_bytes <= ((size_t)64 << 20)) {  // up_bytes is bounded anyway
             g_lanes.push_back(ln);
             ln = Lane();
             return;
@@ -230,6 +244,14 @@ void lane_trim()
     }
     (void)hipSetDevice(cur);
 }
+
+// One fused launch at a time.  Its workgroups wait, while resident, for earlier workgroups of the same
+// launch.  Alone on the device that cannot block: every XCD starts its share of the workgroups in
+// order, so the oldest unfinished one is resident and waits for nothing.  Two such launches side by
+// side can fill an XCD each with workgroups waiting for one that needs a place on the other XCD;
+// the bounded wait then runs out (seconds) and both fall back to per-layer launches.  Launches
+// without such waits (one per layer) may run beside a fused one: their workgroups always finish.
+std::mutex g_fused_mu;
 
 struct HostInst {
     int orig;  // index in the caller's arrays
@@ -332,11 +354,13 @@ struct gdp_plan {
     size_t back_bytes = 0;
     const GdpDevOut *h_out = nullptr;
     const int32_t *h_res = nullptr;
-    std::vector<char> stage;     // host copy of the inputs' device layout; the upload reads it asynchronously
+    std::vector<char> stage;     // host copy of the inputs' device layout when it is too large for lane.up;
+                                 // the upload reads it asynchronously
     double relaxations = 0, relax_bytes = 0;
     double executed = 0;     // relaxations actually carried out (tiles inside the bands)
     bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
     bool ran = false;
+    bool holds_fused = false;     // between run_enqueue and run_finish of a fused run: g_fused_mu is held
     bool fused = true;            // one launch for all layers instead of one per layer
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
@@ -419,8 +443,12 @@ int validate(const gdp_problem *p, int i)
 void destroy(gdp_plan *pl)
 {
     if (!pl) return;
+    if (pl->holds_fused) {  // a run that was started and never waited for
+        pl->holds_fused = false;
+        g_fused_mu.unlock();
+    }
     if (pl->dbase || pl->lane.stream) (void)hipSetDevice(pl->device);
-    if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read pl->stage
+    if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read its host copy
     if (pl->dbase) arena_give(pl->device, pl->dbase, pl->dalloc);
     for (hipEvent_t e : pl->ev_relax) (void)hipEventDestroy(e);
     lane_give(pl->lane);
@@ -745,11 +773,29 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         return fail_hip(e, buf);
     }
     // ---- build the small region on the host ------------------------------------------------------
-    std::vector<char> &stage = pl->stage;
-    try {
-        stage.assign(small_bytes, 0);
-    } catch (const std::bad_alloc &) {
-        return fail(GDP_E_NOMEM, "host staging allocation failed");
+    {
+        const hipError_t e = lane_take(pl->device, pl->back_bytes, small_bytes, &pl->lane);
+        if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
+            (void)hipGetLastError();
+            return fail(GDP_E_NOMEM, "page-locked host memory for inputs and results");
+        }
+        GDP_HIP(e);
+        pl->stream = pl->lane.stream;
+        pl->ev_begin = pl->lane.ev_begin;
+        pl->ev_end = pl->lane.ev_end;
+    }
+    struct { char *p; char *data() const { return p; } } stage = {pl->lane.up};
+    if (small_bytes > UPLOAD_PINNED_MAX) {
+        try {
+            pl->stage.assign(small_bytes, 0);
+        } catch (const std::bad_alloc &) {
+            return fail(GDP_E_NOMEM, "host staging allocation failed");
+        }
+        stage.p = pl->stage.data();
+    } else {
+        // the previous plan of this lane has been destroyed, i.e. its stream waited for: nothing reads
+        // the buffer any more
+        memset(stage.p, 0, small_bytes);
     }
     std::vector<std::vector<int32_t>> h_band((size_t)n);
     GdpDevInst *di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
@@ -905,17 +951,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
-    {
-        const hipError_t e = lane_take(pl->device, pl->back_bytes, &pl->lane);
-        if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
-            (void)hipGetLastError();
-            return fail(GDP_E_NOMEM, "page-locked host memory for the results");
-        }
-        GDP_HIP(e);
-        pl->stream = pl->lane.stream;
-        pl->ev_begin = pl->lane.ev_begin;
-        pl->ev_end = pl->lane.ev_end;
-    }
     GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
@@ -923,13 +958,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, GDP_INIT_PADS | GDP_INIT_ZERO,
                                     pl->stream));
     }
-    // no wait here: the stream orders the upload and these fills before the first run, pl->stage stays
-    // alive as long as the plan, and an error of theirs is reported by the run
+    // no wait here: the stream orders the upload and these fills before the first run, the host copy
+    // stays alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);
     return GDP_OK;
 }
 
-int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
+int run(gdp_plan *pl, int32_t mode, gdp_timing *t);
+
+// Everything of a run that does not wait: the launches and the copy of the results into the plan's
+// page-locked buffer, on the plan's stream.
+int run_enqueue(gdp_plan *pl, int32_t mode)
 {
     GDP_HIP(hipSetDevice(pl->device));
     const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
@@ -952,6 +991,10 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, what, pl->stream));
     }
     size_t li = 0;
+    if (pl->fused && !pl->holds_fused) {
+        g_fused_mu.lock();  // until run_finish has waited for the launch (same thread)
+        pl->holds_fused = true;
+    }
     if (pl->fused) {
         GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
                                 pl->stream));
@@ -981,7 +1024,21 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
     GDP_HIP(hipMemcpyAsync(pl->lane.back, pl->dbase + pl->off_abort, pl->back_bytes, hipMemcpyDeviceToHost,
                            pl->stream));
-    GDP_HIP(hipStreamSynchronize(pl->stream));
+    return GDP_OK;
+}
+
+// Waits for what run_enqueue started; repeats the run with one launch per layer if a fused launch gave up.
+int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
+{
+    GDP_HIP(hipSetDevice(pl->device));
+    size_t launches = 0;
+    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : (size_t)g.max_L;
+    const hipError_t waited = hipStreamSynchronize(pl->stream);
+    if (pl->holds_fused) {
+        pl->holds_fused = false;
+        g_fused_mu.unlock();
+    }
+    GDP_HIP(waited);
     pl->h_out = reinterpret_cast<const GdpDevOut *>(pl->lane.back + (pl->off_out - pl->off_abort));
     pl->h_res = reinterpret_cast<const int32_t *>(pl->lane.back + (pl->off_res - pl->off_abort));
     // the flag is cleared and written by fused launches only
@@ -1023,6 +1080,16 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
         }
     }
     return GDP_OK;
+}
+
+int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
+{
+    const int rc = run_enqueue(pl, mode);
+    if (rc != GDP_OK && pl->holds_fused) {  // a launch failed: nothing to wait for
+        pl->holds_fused = false;
+        g_fused_mu.unlock();
+    }
+    return rc == GDP_OK ? run_finish(pl, mode, t) : rc;
 }
 
 int fetch(gdp_plan *pl, gdp_result *const *r)
@@ -1077,17 +1144,14 @@ int fetch(gdp_plan *pl, gdp_result *const *r)
 
 extern "C" {
 
-int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
+}  // extern "C"
+
+namespace {
+
+// A plan for problems that validate() has accepted.
+int create_checked(int32_t n, const gdp_problem *const *p, gdp_plan **out)
 {
-    g_err.clear();
-    if (!out) return fail(GDP_E_BADARG, "null plan pointer");
     *out = nullptr;
-    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
-    if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
-    for (int i = 0; i < n; ++i) {
-        int rc = validate(p[i], i);
-        if (rc != GDP_OK) return rc;
-    }
     for (int attempt = 0; attempt < 2; ++attempt) {
         gdp_plan *pl = new (std::nothrow) gdp_plan();
         if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
@@ -1105,6 +1169,24 @@ int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
         if (rc != GDP_RETRY_WITH_MARKS || attempt == 1) return rc == GDP_RETRY_WITH_MARKS ? fail(GDP_E_NOMEM, "device memory") : rc;
     }
     return fail(GDP_E_NOMEM, "device memory");
+}
+
+}  // namespace
+
+extern "C" {
+
+int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
+{
+    g_err.clear();
+    if (!out) return fail(GDP_E_BADARG, "null plan pointer");
+    *out = nullptr;
+    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
+    if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
+    for (int i = 0; i < n; ++i) {
+        int rc = validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+    }
+    return create_checked(n, p, out);
 }
 
 int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing)
@@ -1170,7 +1252,8 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
     // memory is solved in consecutive parts that reuse one allocation: the time to obtain device
     // memory grows with its size, the time to solve a part does not grow faster than its share.
     const size_t budget = std::max<size_t>(env_mb("GALVATRON_DP_ARENA_MB", 8192), (size_t)1 << 20);
-    int begin = 0;
+    int begin = 0, prev_begin = 0;
+    gdp_plan *prev = nullptr;
     while (begin < n) {
         int end = begin;
         size_t bytes = 0;
@@ -1180,16 +1263,37 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
             bytes += b;
             ++end;
         }
+        // The next part is laid out and uploaded, and the constant parts of its cost buffers are filled
+        // (on a stream of its own), while the previous part still runs; it is launched as soon as that
+        // one has finished, before that one's results are handed out.
         gdp_plan *pl = nullptr;
-        int rc = gdp_plan_create(end - begin, p + begin, &pl);
-        if (rc != GDP_OK) return rc;
-        rc = run(pl, 0, nullptr);
-        if (rc == GDP_OK) rc = fetch(pl, r + begin);
-        destroy(pl);
-        if (rc != GDP_OK) return rc;
+        int rc = create_checked(end - begin, p + begin, &pl);
+        int rp = prev ? run_finish(prev, 0, nullptr) : GDP_OK;
+        if (rc == GDP_OK && rp == GDP_OK) {
+            rc = run_enqueue(pl, 0);
+            if (rc != GDP_OK && pl->holds_fused) {
+                pl->holds_fused = false;
+                g_fused_mu.unlock();
+            }
+        }
+        if (prev) {
+            if (rp == GDP_OK) rp = fetch(prev, r + prev_begin);
+            destroy(prev);
+            prev = nullptr;
+            if (rc == GDP_OK) rc = rp;
+        }
+        if (rc != GDP_OK) {
+            destroy(pl);
+            return rc;
+        }
+        prev = pl;
+        prev_begin = begin;
         begin = end;
     }
-    return GDP_OK;
+    int rc = run_finish(prev, 0, nullptr);
+    if (rc == GDP_OK) rc = fetch(prev, r + prev_begin);
+    destroy(prev);
+    return rc;
 }
 
 int gdp_solve(const gdp_problem *p, gdp_result *r)

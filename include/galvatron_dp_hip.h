@@ -146,7 +146,7 @@ void gdp_plan_destroy(gdp_plan *plan);
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
 
 /* Frees the device allocations that finished plans left behind for reuse (no counterpart in the
- * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 16384, 0 keeps
+ * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 20480, 0 keeps
  * nothing), because obtaining device memory costs far more than a solve.  Finished plans also leave
  * their stream, two events and page-locked result buffer for the next plan (at most 64 sets; creating
  * and destroying a stream takes a third as long as a small solve); this call releases those too. */

@@ -161,6 +161,42 @@ def test_streams_and_result_buffers_handed_from_plan_to_plan(golden):
         _check_against_golden(prob, golden[n], n)
 
 
+def test_fused_runs_from_several_threads_take_turns(golden):
+    """Workgroups of a fused launch wait for earlier ones of the same launch; two such launches side
+    by side could each fill XCDs that the other needs.  The library lets one fused launch run at a
+    time, so none of them ever has to give up (which would take seconds), whatever the threads do."""
+    import threading
+    import time
+    if os.environ.get("GALVATRON_DP_FUSED") == "0":
+        pytest.skip("the environment presets per-layer launches")
+    names = ["cfg3_smallV_%d" % i for i in range(8)] * 12         # 96 instances: enough blocks to fill the device
+    errors, gave_up = [], []
+
+    def work(k):
+        try:
+            probs = [_problem(H.build_case(golden[n]), launch="fused") for n in names]
+            with _lib.Plan(probs) as plan:
+                plan.set_option(_lib.GDP_OPT_NO_FALLBACK, 1)   # an abandoned launch raises instead of switching
+                for _ in range(6):
+                    t = plan.run(1)
+                    gave_up.append(not t.fused)
+                plan.fetch()
+            for n, prob in zip(names, probs):
+                _check_against_golden(prob, golden[n], f"thread {k} {n}")
+        except Exception as e:  # noqa: BLE001
+            errors.append((k, repr(e)))
+
+    t0 = time.perf_counter()
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert not any(gave_up)
+    assert time.perf_counter() - t0 < 30
+
+
 @pytest.mark.parametrize("chunk,max_rows", [(1, 65535), (3, 65535), (2, 5), (1000, 3), (4, 1)])
 def test_instances_taken_through_the_launch_a_few_at_a_time(golden, monkeypatch, chunk, max_rows):
     """A fused launch takes `chunk` instances at a time through all their layers (grid rows follow a
