@@ -274,10 +274,15 @@ struct Group {  // instances with the same S, sorted by L descending
     struct Segment { int first, layers; unsigned lds_bytes; };
     std::vector<Segment> segments;  // fused launches: runs of layers with the same active set, or -- chunked --
                                     // runs of at most 65535 entries of the row table
+    bool latency = false;           // per-layer launches use the variant for launches with few waves
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
     std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
     size_t off_rows = 0;
     GdpSched sched = {};      // argument of the fused launches (device pointers inside)
+    bool latency_possible(bool keep_marks) const
+    {
+        return !keep_marks && GDP_VARIANTS[variant].ts == GDP_LAT_TS && GDP_VARIANTS[variant].r == GDP_LAT_R;
+    }
     size_t off_active, off_cnt, off_lay;  // byte offsets in the device allocation
 };
 
@@ -376,6 +381,7 @@ struct gdp_plan {
     int occupancy_cap_override = 0; // GALVATRON_DP_OCCUPANCY_CAP=n: n workgroups per CU in fused launches
     int chunk_override = 0;         // GALVATRON_DP_CHUNK=n: n instances at a time in fused launches
     int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
+    int latency_override = -1;  // GALVATRON_DP_LATENCY_VARIANT=0|1: never / wherever it exists (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
 
@@ -533,6 +539,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
+    if (const char *e = getenv("GALVATRON_DP_LATENCY_VARIANT")) pl->latency_override = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_CHUNK")) pl->chunk_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) {
         pl->no_occupancy_cap = atoi(e) == 0;
@@ -590,9 +597,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         int j = i;
         while (j < n && inst[(size_t)j].S == g.S) ++j;
         g.count = j - i;
-        // Register tile.  Width: least padding of S.  Height: the tallest whose first layer still
-        // gives every resident wave at least two tasks, so that the stores of one task drain under
-        // the arithmetic of the next; small problems get the shortest (most parallel) one.
+        // Register tile.  Width: pick_ts.  Height: the tallest whose first layer still gives every
+        // resident wave at least two tasks, so that the stores of one task drain under the arithmetic
+        // of the next; small problems get the shortest (most parallel) one.
         int64_t tiles64 = 0;
         for (int k = i; k < j; ++k) tiles64 += ((int64_t)inst[(size_t)k].V + 63) / 64;
         const int ts = pick_ts(g.S, pl->keep_marks, tiles64, wave_slots);
@@ -686,6 +693,18 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             }
         }
         pl->fused = first_layer * (all > 0 ? live / all : 1.0) >= 2.0 * pl->num_cu;
+    }
+    // Launches that small run one or two waves per SIMD, and what they wait for is memory latency, not
+    // instruction issue: their narrowest tile has a variant built for that (measured, 16 layers, one
+    // instance: S=22 V=16384 0.176 -> 0.126 ms, S=44 V=16384 0.241 -> 0.208, S=64 V=4096 0.284 -> 0.192;
+    // with all layers in one launch, or on larger problems, it is the slower one).
+    for (Group &g : pl->groups) {
+        const GdpVariant &v = GDP_VARIANTS[g.variant];
+        g.latency = !pl->fused && !pl->keep_marks && v.ts == GDP_LAT_TS && v.r == GDP_LAT_R;
+        if (pl->latency_override >= 0) g.latency = g.latency_possible(pl->keep_marks) && pl->latency_override != 0;
+        if (g.latency)
+            for (int k = g.first; k < g.first + g.count; ++k)
+                inst[(size_t)k].SU = (int)align_up((size_t)inst[(size_t)k].S, GDP_SRC_UNROLL_LAT);
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -1013,7 +1032,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             for (const Group &g : pl->groups) {
                 if (l >= g.max_L) continue;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks,
+                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, g.latency && !pl->keep_marks,
                                          reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
                                          g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
@@ -1066,6 +1085,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
             t->tile_ts = GDP_VARIANTS[g0.variant].ts;
             t->tile_r = GDP_VARIANTS[g0.variant].r;
             t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
+            t->latency_variant = (!pl->fused && g0.latency) ? 1 : 0;
         }
         t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));

@@ -44,7 +44,8 @@
 #define GDP_WAVES_PER_BLOCK 4
 #endif
 #define GDP_SRC_UNROLL 4  // source strategies are consumed up to four per trip (padded with +inf sources)
-#define GDP_SRC_PAD 8     // dummy source rows after SU in roff / inter: targets of the last prefetches
+#define GDP_SRC_PAD 16    // dummy source rows after SU in roff / inter: targets of the last prefetches
+#define GDP_SRC_UNROLL_LAT 8  // sources per trip of the latency variant (its groups pad S to this)
 
 struct GdpDevInst {
     double *H;        // buffer b starts at H + b * hstride
@@ -58,7 +59,7 @@ struct GdpDevInst {
     int64_t ld;          // elements per row of H
     int64_t ldm;         // entries per row of M
     int32_t L, V, S, SP;
-    int32_t SU;     // S rounded up to GDP_SRC_UNROLL
+    int32_t SU;     // S rounded up to GDP_SRC_UNROLL (GDP_SRC_UNROLL_LAT where the latency variant runs)
     int32_t P;      // +inf elements in front of every H row
     int32_t ntile;  // row tiles covering [0, V)
     int32_t nbuf;
@@ -131,8 +132,12 @@ static const GdpVariant GDP_VARIANTS[] = {
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
 // marks: track and store the argmin table (otherwise costs only).  lay: the group's table of
 // n_inst x max_L records.
-hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile,
-                            int SP, int layer, hipStream_t stream);
+// latency: the variant for launches too small to hide memory latency behind other waves (costs only,
+// tile GDP_LAT_TS x GDP_LAT_R, SU a multiple of GDP_SRC_UNROLL_LAT); see relax_task_lat.
+hipError_t gdp_launch_relax(int variant, bool marks, bool latency, const GdpDevLayer *lay, int max_L, int n_inst,
+                            int max_ntile, int SP, int layer, hipStream_t stream);
+#define GDP_LAT_TS 8
+#define GDP_LAT_R 1
 // Layers layer0 .. layer0+layers-1 of a group in one launch (grid = block tasks of a layer x
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
 // lds_bytes: dynamic LDS per workgroup, unused by the kernel; it limits how many workgroups a CU holds.

@@ -91,6 +91,136 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
         }
 }
 
+// relax_task for launches with too few waves to hide memory latency (costs only, per-layer launches).
+// In relax_task every step waits for a scalar load issued one step earlier (the next row of transition
+// costs; scalar loads return out of order, so there is no waiting for "all but the latest"), about
+// 0.2 us when it misses the scalar cache -- nothing when other waves fill the gap, the whole run time
+// of a layer when there are one or two waves per SIMD.  Here nothing inside a trip waits for a
+// scalar load:
+//   - the row of transition costs travels as a vector load (lane j holds column j), NS steps ahead
+//     like the cost rows -- vector loads return in order, so a wait can leave the younger ones in
+//     flight -- and is spread to scalar registers with v_readlane (2*TS more vector instructions per
+//     step; instruction issue is not what such a launch is short of);
+//   - the row offsets of a whole trip are fetched with the previous trip's.
+// Same arithmetic in the same order as relax_task, hence the same bits.
+template <int TS, int R, bool PUBLISH>
+__device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
+{
+    constexpr int NS = 8;
+    static_assert(GDP_SRC_UNROLL_LAT % NS == 0 && GDP_SRC_PAD >= 2 * NS, "padding of roff / inter");
+    const int SU = uload(&Y->SU);   // a multiple of NS in the groups this variant runs for
+    const int SP = uload(&Y->SP);
+    const double *src = uload(&Y->src);
+    const int64_t *ro = uload(&Y->ro);
+    const int s0 = tb * TS;
+    const double *it = uload(&Y->it) + s0;
+    const int64_t u0 = (int64_t)tile * (64 * R);
+    const unsigned lane_bytes = lane * 8u;
+    const unsigned col_bytes = (lane < (unsigned)TS ? lane : (unsigned)(TS - 1)) * 8u;
+
+    double best[R][TS];
+    int arg_unused[1][1];
+    double add_unused[TS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < TS; ++j) best[r][j] = INFINITY;
+#pragma unroll
+    for (int j = 0; j < TS; ++j) add_unused[j] = 0.0;
+
+    double fp[NS][R], scv[NS];
+    int64_t ocur[NS], onext[NS];
+    const double *itp = it;   // row of the transition matrix that the next request fetches
+    {
+        int64_t o0[NS];
+#pragma unroll
+        for (int u = 0; u < NS; ++u) o0[u] = uload(ro + u);
+#pragma unroll
+        for (int u = 0; u < NS; ++u) ocur[u] = uload(ro + NS + u);
+        GDP_SCHED_FENCE();
+        unsigned lb = lane_bytes, cb = col_bytes;
+        GDP_PIN_LANE(lb);
+        GDP_PIN_LANE(cb);
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            const double *p = src + o0[u] + u0;
+            asm volatile("" : "+s"(p));
+#pragma unroll
+            for (int r = 0; r < R; ++r) fp[u][r] = lane_load(p, lb, r);
+            const double *q = itp;
+            asm volatile("" : "+s"(q));
+            scv[u] = lane_load(q, cb, 0);
+            itp += SP;
+            GDP_SCHED_FENCE();
+        }
+    }
+    const int64_t *rop = ro + 2 * NS;
+    for (int sp = 0; sp < SU; sp += NS) {
+        unsigned lb = lane_bytes, cb = col_bytes;
+        GDP_PIN_LANE(lb);
+        GDP_PIN_LANE(cb);
+        // row offsets for the requests of the next trip: a whole trip ahead of their use
+#pragma unroll
+        for (int u = 0; u < NS; ++u) onext[u] = uload(rop + u);
+        GDP_SCHED_FENCE();
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            double sc[TS];
+            {
+                const int lo = __double2loint(scv[u]), hi = __double2hiint(scv[u]);
+#pragma unroll
+                for (int j = 0; j < TS; ++j)
+                    sc[j] = __hiloint2double(__builtin_amdgcn_readlane(hi, j), __builtin_amdgcn_readlane(lo, j));
+            }
+            relax_cols<TS, R, false, 0, TS>(best, arg_unused, fp[u], sc, add_unused, sp + u);
+            GDP_SCHED_FENCE();
+            {
+                const double *pn = src + ocur[u] + u0;
+                asm volatile("" : "+s"(pn));
+#pragma unroll
+                for (int r = 0; r < R; ++r) fp[u][r] = lane_load(pn, lb, r);
+                const double *q = itp;
+                asm volatile("" : "+s"(q));
+                scv[u] = lane_load(q, cb, 0);
+                itp += SP;
+            }
+            GDP_SCHED_FENCE();
+        }
+#pragma unroll
+        for (int u = 0; u < NS; ++u) ocur[u] = onext[u];
+        rop += NS;
+    }
+
+    const GdpDevLayer *Z = Y;
+    asm volatile("" : "+s"(Z));
+    {
+        const double *iz = uload(&Z->ia) + s0;
+#pragma unroll
+        for (int j = 0; j < TS; ++j) {
+            const double a = uload(iz + j);
+#pragma unroll
+            for (int r = 0; r < R; ++r) best[r][j] += a;
+        }
+    }
+    const int64_t ld = uload(&Z->ld);
+    const int nvalid = uload(&Z->S) - s0;
+    double *drow = uload(&Z->dst) + (int64_t)s0 * ld + u0;
+#pragma unroll
+    for (int j = 0; j < TS; ++j) {
+        if (j < nvalid) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (PUBLISH)
+                    __hip_atomic_store(drow + (lane + 64u * r), best[r][j], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    drow[lane + 64u * r] = best[r][j];
+            }
+            drow += ld;
+        }
+    }
+}
+
 // One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of the layer described
 // by Y.
 // PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
@@ -290,7 +420,7 @@ __device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, 
 // ---- one launch per layer ------------------------------------------------------------------------
 // __launch_bounds__: register allocation is held to 16 resident waves per CU (4 per SIMD, at most
 // 128 VGPRs).
-template <int TS, int R, bool ARG>
+template <int TS, int R, bool ARG, bool LAT = false>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
     const GdpDevLayer *__restrict__ lay, int max_L, int layer, unsigned ntb)
 {
@@ -308,7 +438,10 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         if (task >= live_tasks) return;
         const unsigned t = task / ntb;
-        relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
+        if constexpr (LAT)
+            relax_task_lat<TS, R, false>(Y, (unsigned)lo + t, task - t * ntb, lane);
+        else
+            relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
     } else {
         const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         const unsigned t = task / ntb;
@@ -731,7 +864,7 @@ __global__ __launch_bounds__(256) void gdp_export_mark_kernel(const GdpDevInst *
 
 }  // namespace
 
-template <int TS, int R, bool ARG>
+template <int TS, int R, bool ARG, bool LAT = false>
 static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile_rows, int SP, int layer,
                                  hipStream_t stream)
 {
@@ -740,7 +873,7 @@ static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, 
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     nblk = ((nblk + 7u) & ~7u) + 8u;  // live blocks are rounded up to 8, the fill blocks come after them
     dim3 grid(nblk, (unsigned)n_inst, 1), block(64 * GDP_WAVES_PER_BLOCK, 1, 1);
-    hipLaunchKernelGGL((gdp_relax_kernel<TS, R, ARG>), grid, block, 0, stream, lay, max_L, layer, ntb);
+    hipLaunchKernelGGL((gdp_relax_kernel<TS, R, ARG, LAT>), grid, block, 0, stream, lay, max_L, layer, ntb);
     return hipGetLastError();
 }
 
@@ -780,9 +913,15 @@ static hipError_t launch_fused_v(bool marks, dim3 grid, dim3 block, unsigned lds
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_relax(int variant, bool marks, const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile,
-                            int SP, int layer, hipStream_t stream)
+hipError_t gdp_launch_relax(int variant, bool marks, bool latency, const GdpDevLayer *lay, int max_L, int n_inst,
+                            int max_ntile, int SP, int layer, hipStream_t stream)
 {
+    if (latency) {
+        if (marks || variant < 0 || variant >= GDP_NUM_VARIANTS || GDP_VARIANTS[variant].ts != GDP_LAT_TS ||
+            GDP_VARIANTS[variant].r != GDP_LAT_R)
+            return hipErrorInvalidValue;
+        return launch_relax_t<GDP_LAT_TS, GDP_LAT_R, false, true>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+    }
 #define X(id, ts, r, m) \
     case id: return launch_relax_v<ts, r, m>(marks, lay, max_L, n_inst, max_ntile, SP, layer, stream);
     switch (variant) {

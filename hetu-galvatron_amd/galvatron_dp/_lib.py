@@ -62,7 +62,8 @@ class gdp_timing(ctypes.Structure):
     _fields_ = [("total_ms", ctypes.c_float), ("relax_ms", ctypes.c_float), ("relax_launches", ctypes.c_int32),
                 ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("executed", ctypes.c_double),
                 ("relax_bytes", ctypes.c_double), ("tile_ts", ctypes.c_int32), ("tile_r", ctypes.c_int32),
-                ("keep_marks", ctypes.c_int32), ("chunk", ctypes.c_int32)]
+                ("keep_marks", ctypes.c_int32), ("chunk", ctypes.c_int32),
+                ("latency_variant", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 _lib = None

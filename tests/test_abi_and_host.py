@@ -30,7 +30,7 @@ def test_version_and_struct_sizes():
     assert _lib.lib().gdp_version() == 100
     assert ctypes.sizeof(_lib.gdp_problem) == 80
     assert ctypes.sizeof(_lib.gdp_result) == 40
-    assert ctypes.sizeof(_lib.gdp_timing) == 56
+    assert ctypes.sizeof(_lib.gdp_timing) == 64
 
 
 def test_validation_happens_before_any_device_work():

@@ -161,6 +161,37 @@ def test_streams_and_result_buffers_handed_from_plan_to_plan(golden):
         _check_against_golden(prob, golden[n], n)
 
 
+@pytest.mark.parametrize("S", [1, 7, 8, 9, 15, 16, 17, 40, 44, 63, 100])
+def test_small_launches_use_the_latency_variant(S, monkeypatch):
+    """One small instance, one launch per layer: the narrowest tile runs in the variant that keeps
+    scalar loads out of its loop (sources padded to 8 per trip, transition costs spread from a vector
+    register).  Same bits as the ordinary variant and as the oracle, f included; S on both sides of
+    the trip length and of the tile width."""
+    if any(k in os.environ for k in ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R",
+                                     "GALVATRON_DP_FUSED", "GALVATRON_DP_LATENCY_VARIANT")):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    rng = np.random.Generator(np.random.PCG64([3, S]))
+    inst = W.random_instance(rng, 5, S, 700 + S, mem_hi=150, inf_frac=0.1, per_layer_inter=bool(S % 2), n_keys=3)
+    wt, wr, wm, wf, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+    keys = sorted(inst.other_mem)
+    seen = []
+    for preset in (None, "0"):
+        if preset is not None:
+            monkeypatch.setenv("GALVATRON_DP_LATENCY_VARIANT", preset)
+        prob = _problem(inst, export_f=True)
+        with _lib.Plan([prob]) as plan:
+            plan.set_option(_lib.GDP_OPT_POISON, 1)
+            t = plan.run(1)
+            plan.fetch()
+        seen.append((t.fused, t.tile_ts, t.tile_r, t.latency_variant))
+        got = ({k: prob.total[i] for i, k in enumerate(keys)}, {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+               {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+        H.assert_same_results(got, (wt, wr, wm), f"S={S} preset={preset}")
+        assert prob.f_out.tobytes() == wf.tobytes()
+    assert seen == [(0, 8, 1, 1), (0, 8, 1, 0)]
+
+
 def test_fused_runs_from_several_threads_take_turns(golden):
     """Workgroups of a fused launch wait for earlier ones of the same launch; two such launches side
     by side could each fill XCDs that the other needs.  The library lets one fused launch run at a

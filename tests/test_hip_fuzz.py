@@ -48,7 +48,7 @@ def _compare(inst, tag, launch=None):
 
 
 @pytest.mark.parametrize("n,shape", list(enumerate(SHAPES)))
-def test_random_instances_against_oracle(n, shape):
+def test_random_instances_against_oracle(n, shape, monkeypatch):
     L, S, V = shape
     if S > _lib.GDP_MAX_S_MARKS and os.environ.get("GALVATRON_DP_KEEP_MARKS", "0") != "0":
         pytest.skip("the environment forces the argmin table, whose entries are bytes")
@@ -59,11 +59,16 @@ def test_random_instances_against_oracle(n, shape):
         inst = W.random_instance(rng, L, S, V, integer_costs=ties, mem_hi=hi, per_layer_inter=bool(variant % 2),
                                  inf_frac=0.2 if variant >= 2 else 0.0, over_frac=0.1 if variant == 3 else 0.0,
                                  n_keys=min(4, 1 + variant))
+        # small per-layer launches use a kernel variant of their own; variant 2 runs without it
+        if variant == 2 and "GALVATRON_DP_LATENCY_VARIANT" not in os.environ:
+            monkeypatch.setenv("GALVATRON_DP_LATENCY_VARIANT", "0")
         _compare(inst, f"shape {shape} variant {variant}", launch=("fused", "per_layer", None, None)[variant])
+        if variant == 2:
+            monkeypatch.undo()
 
 
 @pytest.mark.parametrize("shape", [(4, 8, 300), (3, 16, 200), (5, 11, 257), (3, 64, 150), (2, 44, 129)])
-def test_candidates_that_collide_only_after_the_intra_addition(shape):
+def test_candidates_that_collide_only_after_the_intra_addition(shape, monkeypatch):
     """Transition costs that differ in the last bits under intra costs some 2^40 times larger: many
     candidates (f + inter) + intra are then EQUAL although their (f + inter) differ, so the reference's
     lowest-index rule picks a source that is not the one with the smallest f + inter.  The costs-only
@@ -87,6 +92,9 @@ def test_candidates_that_collide_only_after_the_intra_addition(shape):
     assert differs > 0
     for launch in ("fused", "per_layer"):
         _compare(inst, f"collisions {shape} {launch}", launch=launch)
+    if "GALVATRON_DP_LATENCY_VARIANT" not in os.environ:
+        monkeypatch.setenv("GALVATRON_DP_LATENCY_VARIANT", "0")    # the ordinary variant of the narrowest tile
+        _compare(inst, f"collisions {shape} per_layer, ordinary variant", launch="per_layer")
 
 
 def test_no_keys_and_single_layer():
