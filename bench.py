@@ -166,12 +166,15 @@ def main() -> int:
             "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
             "device_ms": t1.total_ms, "executed_fraction": tm.executed / relax,
             "tflops": 3.0 * tm.executed / launches / avg_launch_s / 1e12,
-            "issued_per_relaxation": 5.0 if keep_marks else 2.0 + 1.0 / insts[0].S,
+            # the variant for small per-layer launches spends two more vector instructions per relaxation on
+            # spreading the transition costs from a vector register (v_readlane)
+            "issued_per_relaxation": 5.0 if keep_marks else (4.0 if tm.latency_variant else 2.0) + 1.0 / insts[0].S,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
             "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
             "tile": "%d target strategies x %d budget rows per wavefront" % (tm.tile_ts, 64 * tm.tile_r),
-            "kernel": "gdp_relax_fused_kernel" if tm.fused else "gdp_relax_kernel",
+            "kernel": "gdp_relax_fused_kernel" if tm.fused else
+                      ("gdp_relax_kernel (latency variant)" if tm.latency_variant else "gdp_relax_kernel"),
         }
 
     m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping)
