@@ -27,6 +27,9 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    the backtrack recomputes the argmin of the L cells on its path.  ``with_mark_table``
                    reports the mode that stores the reference's argmin table instead: 17 bytes and
                    five instead of two vector instructions per relaxation).
+* ``config.search_wall_ms_from_host_arrays``  the same solve through gdp_solve_batch from host arrays
+                   (validation, layout, upload, all kernels, download; median of a few calls), beside
+                   ``search_wall_ms_device`` (first kernel to last kernel of one solve, HIP events).
 * ``cpu_baseline`` the reference's own dp_core (compiled into oracle/_ref by oracle/build.py) or,
                    where that file is absent, the C restatement in oracle/, timed on this host on a
                    bounded sample of the same workload (its first layers), one thread.
@@ -144,7 +147,7 @@ def main() -> int:
         print(json.dumps({"calibrate_copy_bytes": n, "copies": 3}))
         return 0
 
-    def measure(workload, steps, warmup, compute_all=True, keep_marks=False):
+    def measure(workload, steps, warmup, compute_all=True, keep_marks=False, host_leg=False):
         insts, probs = _problems(workload, compute_all, keep_marks)
         with _lib.Plan(probs) as plan:
             for _ in range(warmup):
@@ -158,13 +161,21 @@ def main() -> int:
             tm = plan.run(2)                       # per-launch HIP events on the plan's stream
             t1 = plan.run(1)
             plan.fetch()
+        # The same solve from host arrays through gdp_solve_batch: validation, layout, upload, all kernels,
+        # download (device memory of earlier calls is reused).  Reported beside the headline, never as it.
+        host_ms = []
+        for _ in range(1 + max(3, min(steps, 5)) if host_leg else 0):
+            h0 = time.perf_counter()
+            _lib.solve_batch(probs)
+            host_ms.append((time.perf_counter() - h0) * 1e3)
+        host_ms = sorted(host_ms[1:])[len(host_ms[1:]) // 2] if host_leg else None
         relax = tm.relaxations
         launches = tm.relax_launches
         avg_launch_s = tm.relax_ms * 1e-3 / launches
         return {
             "insts": insts, "probs": probs, "relaxations": relax, "ms_per_step": wall / steps * 1e3,
             "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
-            "device_ms": t1.total_ms, "executed_fraction": tm.executed / relax,
+            "device_ms": t1.total_ms, "host_ms": host_ms, "executed_fraction": tm.executed / relax,
             "tflops": 3.0 * tm.executed / launches / avg_launch_s / 1e12,
             # the variant for small per-layer launches spends two more vector instructions per relaxation on
             # spreading the transition costs from a vector register (v_readlane)
@@ -177,7 +188,7 @@ def main() -> int:
                       ("gdp_relax_kernel (latency variant)" if tm.latency_variant else "gdp_relax_kernel"),
         }
 
-    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping)
+    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping, host_leg=not a.headline_only)
     insts = m["insts"]
     first = insts[0]
     traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(a.workload + ("+row_skipping" if a.row_skipping else ""))
@@ -187,7 +198,8 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
-                   "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"], "launch_scheme": m["scheme"],
+                   "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"],
+                   "search_wall_ms_from_host_arrays": m["host_ms"], "launch_scheme": m["scheme"],
                    "register_tile": m["tile"],
                    "relaxations_executed_fraction": m["executed_fraction"], "device": _lib.device_info()},
         "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
@@ -202,8 +214,9 @@ def main() -> int:
     }
     also = {}
     for w in [x for x in a.also.split(",") if x and x != a.workload]:
-        mm = measure(w, max(3, a.steps // 4), 1)
+        mm = measure(w, max(3, a.steps // 4), 1, host_leg=not a.headline_only)
         also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
+                   "search_wall_ms_from_host_arrays": mm["host_ms"],
                    "launch_scheme": mm["scheme"],
                    "roofline_frac_valu_fp64": mm["tflops"] / PEAK_FP64_VALU_TFLOPS,
                    "roofline_frac_hbm": mm["gbs"] / PEAK_HBM_GBS, "avg_launch_ms": mm["avg_launch_ms"]}
