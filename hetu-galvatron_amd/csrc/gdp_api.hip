@@ -916,6 +916,24 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         sc->n_active = reinterpret_cast<const int32_t *>(pl->dbase + g.off_active);
         sc->max_L = g.max_L; sc->max_ntile = g.max_ntile; sc->ntb = g.ntb;
         sc->group = g.xcd_group;
+        if (!pl->keep_marks) {
+            // Costs only: a fused launch holds the block tasks of the bands alone (the rows below a
+            // band are filled once, below; the rows above it are never read).  Slots per XCD: the widest
+            // band of the group, counted in groups of whole tiles from the group its first tile is in.
+            int64_t widest = 1;
+            for (int k = 0; k < g.count; ++k) {
+                const HostInst &h = inst[(size_t)(g.first + k)];
+                for (int l = 0; l < h.L; ++l) {
+                    const int64_t lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
+                    const int64_t hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
+                    if (hi < lo) continue;
+                    const int64_t bt_lo = lo * g.ntb / GDP_WAVES_PER_BLOCK;
+                    const int64_t bt_hi = ((hi + 1) * g.ntb - 1) / GDP_WAVES_PER_BLOCK;
+                    widest = std::max(widest, bt_hi / g.xcd_group - bt_lo / g.xcd_group + 1);
+                }
+            }
+            g.slots = (int)((widest + 7) / 8 * g.xcd_group);
+        }
         sc->slots = g.slots;
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
@@ -974,8 +992,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
         for (const Group &g : pl->groups)
-            GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, GDP_INIT_PADS | GDP_INIT_ZERO,
-                                    pl->stream));
+            GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                    64 * GDP_VARIANTS[g.variant].r,
+                                    GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
     }
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
@@ -1004,10 +1023,13 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
         }
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_begin, pl->stream));
     {
-        const int what = (pl->rezero ? GDP_INIT_ZERO : 0) | (pl->poison ? GDP_INIT_POISON : 0);
+        // (the poison would cover the rows that are filled once per plan: they are filled again after it)
+        const int what = (pl->rezero ? GDP_INIT_ZERO : 0) | (pl->poison ? GDP_INIT_POISON : 0) |
+                         (pl->poison && !pl->keep_marks ? GDP_INIT_FILL : 0);
         if (what)
             for (const Group &g : pl->groups)
-                GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, 0, what, pl->stream));
+                GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                        64 * GDP_VARIANTS[g.variant].r, what, pl->stream));
     }
     size_t li = 0;
     if (pl->fused && !pl->holds_fused) {

@@ -146,12 +146,16 @@ hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched
                                   int layers, unsigned lds_bytes, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
-// in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up).
+// in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up);
+// GDP_INIT_FILL (one cost buffer per layer only): +inf in the rows of layer l's output below its
+// first tile with arithmetic, lay[i * max_L + l].lo (every source cell of those rows is +inf, so the
+// cells are +inf whatever the costs: written once per plan, the costs-only kernels leave them alone).
 #define GDP_INIT_PADS 1
 #define GDP_INIT_ZERO 2
 #define GDP_INIT_POISON 4
-hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, int max_nbuf, int what,
-                           hipStream_t stream);
+#define GDP_INIT_FILL 8
+hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                           int max_L, int tile_rows, int what, hipStream_t stream);
 // Fills n int32 with zero (queue counters; a kernel rather than a memset so that it can be captured).
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream);
 // argmin over the last layer's row + backtrack, one wavefront per key (marks: through the stored

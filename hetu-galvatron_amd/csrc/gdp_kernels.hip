@@ -411,10 +411,12 @@ __device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, 
                                           unsigned lane)
 {
     if ((int)tile > hi) return;
-    if ((int)tile < lo)
-        fill_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
-    else
+    if ((int)tile < lo) {
+        // costs only: every layer has a buffer of its own, and these rows were filled when the plan was made
+        if constexpr (ARG) fill_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
+    } else {
         relax_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
+    }
 }
 
 // ---- one launch per layer ------------------------------------------------------------------------
@@ -442,7 +444,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
             relax_task_lat<TS, R, false>(Y, (unsigned)lo + t, task - t * ntb, lane);
         else
             relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
-    } else {
+    } else if constexpr (ARG) {  // (costs only: those rows were filled when the plan was made)
         const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         const unsigned t = task / ntb;
         const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
@@ -569,13 +571,25 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     // layer before -- was handed out a whole layer earlier on every XCD.
     const unsigned G = (unsigned)Q.group;
     const unsigned grp = w / G;
-    const unsigned bt = (grp * 8u + xcd) * G + (w - grp * G);
-    if (bt >= nbt) return;
+    unsigned bt = (grp * 8u + xcd) * G + (w - grp * G);
     bool live = false;
-    if (hi >= lo) {
+    if constexpr (ARG) {
+        if (bt >= nbt) return;
+        if (hi >= lo) {
+            const unsigned bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
+            const unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
+            live = bt >= bt_lo && bt <= bt_hi;   // carries arithmetic; the others only fill or count as done
+        }
+    } else {
+        // Costs only: the rows below the band were filled when the plan was made and the rows above
+        // it are never read, so only the band's block tasks exist: the slots count from the band's
+        // first group of whole tiles, and a reader waits for tiles of the previous band only.
+        if (hi < lo) return;
         const unsigned bt_lo = ((unsigned)lo * ntb) / GDP_WAVES_PER_BLOCK;
         const unsigned bt_hi = (((unsigned)hi + 1u) * ntb - 1u) / GDP_WAVES_PER_BLOCK;
-        live = bt >= bt_lo && bt <= bt_hi;   // carries arithmetic; the others only fill or count as done
+        bt += bt_lo / G * G;
+        if (bt < bt_lo || bt > bt_hi || bt >= nbt) return;
+        live = true;
     }
     int32_t *cnt_all = Q.cnt;
     // touch what the task reads first (row offsets, first transition costs), so that it sits in the
@@ -599,7 +613,12 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
             int t_hi = (int)((q0 + GDP_WAVES_PER_BLOCK - 1) / ntb);
             if (t_hi >= ntile) t_hi = ntile - 1;
             const int d = uload(&Y[-1].dep);
-            const int first = t_lo - d < 0 ? 0 : t_lo - d;
+            int first = t_lo - d < 0 ? 0 : t_lo - d;
+            if constexpr (!ARG) {  // tiles outside the previous band have no counter to wait for
+                const int plo = uload(&Y[-1].lo), phi = uload(&Y[-1].hi);
+                if (first < plo) first = plo;
+                if (t_hi > phi) t_hi = phi;
+            }
             const bool ok = wait_tiles(cnt_all + ((int64_t)ii * max_L + (layer - 1)) * max_ntile, first, t_hi, (int)ntb,
                                        lane, Q.abort_flag, Q.spin_limit);
             if (lane == 0) sh_ok = ok ? 1 : 0;
@@ -613,7 +632,8 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned tb = q - tile * ntb;
     if (tile >= (unsigned)ntile) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");    // keeps the tile's loads after the wait
-    tile_task<TS, R, true, ARG>(Y, lo, hi, tile, tb, lane);   // tiles outside the band still count as done
+    tile_task<TS, R, true, ARG>(Y, lo, hi, tile, tb, lane);   // with the argmin table: tiles outside the band
+                                                              // are filled or skipped there and count as done
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every write-through store acknowledged
     if (lane == 0)
@@ -628,9 +648,12 @@ __global__ __launch_bounds__(256) void gdp_zero_kernel(int32_t *p, int64_t n)
 }
 
 // Fills of the cost buffers (see GDP_INIT_* in gdp_kernels.h).  grid = (x chunks, rows 0..S, instances).
-__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts, int what)
+__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts,
+                                                       const GdpDevLayer *__restrict__ lay, int max_L, int tile_rows,
+                                                       int what)
 {
     const GdpDevInst *I = insts + blockIdx.z;
+    const GdpDevLayer *Y = lay + (int64_t)blockIdx.z * max_L;
     const int S = uload(&I->S);
     const int row = blockIdx.y;
     if (row > S) return;
@@ -650,6 +673,9 @@ __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restr
             if (what & GDP_INIT_ZERO) h[i] = 0.0;
             if (what & GDP_INIT_POISON)
                 for (int b = 1; b < nbuf; ++b) h[(int64_t)b * hstride + i] = nan;
+            if (what & GDP_INIT_FILL)  // buffer b holds the output of layer b - 1
+                for (int b = 1; b < nbuf; ++b)
+                    if (i - P < (int64_t)uload(&Y[b - 1].lo) * tile_rows) h[(int64_t)b * hstride + i] = inf;
         }
     }
 }
@@ -953,14 +979,13 @@ hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, int max_nbuf, int what,
-                           hipStream_t stream)
+hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                           int max_L, int tile_rows, int what, hipStream_t stream)
 {
-    (void)max_nbuf;
     unsigned bx = (unsigned)((max_ld + 256 * 8 - 1) / (256 * 8));
     if (bx == 0) bx = 1;
     dim3 grid(bx, (unsigned)(max_S + 1), (unsigned)n_inst), block(256, 1, 1);
-    hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts, what);
+    hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts, lay, max_L, tile_rows, what);
     return hipGetLastError();
 }
 
