@@ -56,7 +56,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     "cfg2": 12.131e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
     "cfg3": 45.8e9,     # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
-    "cfg2+row_skipping": 8.641e9,   # profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt
+    "cfg2+row_skipping": 7.652e9,   # profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt
 }
 
 
