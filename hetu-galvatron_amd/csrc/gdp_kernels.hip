@@ -648,12 +648,24 @@ __global__ __launch_bounds__(256) void gdp_zero_kernel(int32_t *p, int64_t n)
 }
 
 // Fills of the cost buffers (see GDP_INIT_* in gdp_kernels.h).  grid = (x chunks, rows 0..S, instances).
-__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts,
-                                                       const GdpDevLayer *__restrict__ lay, int max_L, int tile_rows,
-                                                       int what)
+// GDP_INIT_FILL: grid = (x chunks, rows 0..S-1, instances x layers); buffer l + 1 holds the output of layer l.
+__global__ __launch_bounds__(256) void gdp_fill_kernel(const GdpDevInst *__restrict__ insts,
+                                                       const GdpDevLayer *__restrict__ lay, int max_L, int tile_rows)
+{
+    const int inst = blockIdx.z / max_L, l = blockIdx.z - inst * max_L;
+    const GdpDevInst *I = insts + inst;
+    if (l >= uload(&I->L) || (int)blockIdx.y >= uload(&I->S)) return;
+    int64_t n = (int64_t)uload(&lay[(int64_t)inst * max_L + l].lo) * tile_rows;
+    const int64_t ldm = uload(&I->ldm);
+    if (n > ldm) n = ldm;
+    double *h = uload(&I->H) + (int64_t)(l + 1) * uload(&I->hstride) + (int64_t)blockIdx.y * uload(&I->ld) + uload(&I->P);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        h[i] = INFINITY;
+}
+
+__global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts, int what)
 {
     const GdpDevInst *I = insts + blockIdx.z;
-    const GdpDevLayer *Y = lay + (int64_t)blockIdx.z * max_L;
     const int S = uload(&I->S);
     const int row = blockIdx.y;
     if (row > S) return;
@@ -673,9 +685,6 @@ __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restr
             if (what & GDP_INIT_ZERO) h[i] = 0.0;
             if (what & GDP_INIT_POISON)
                 for (int b = 1; b < nbuf; ++b) h[(int64_t)b * hstride + i] = nan;
-            if (what & GDP_INIT_FILL)  // buffer b holds the output of layer b - 1
-                for (int b = 1; b < nbuf; ++b)
-                    if (i - P < (int64_t)uload(&Y[b - 1].lo) * tile_rows) h[(int64_t)b * hstride + i] = inf;
         }
     }
 }
@@ -985,7 +994,17 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
     unsigned bx = (unsigned)((max_ld + 256 * 8 - 1) / (256 * 8));
     if (bx == 0) bx = 1;
     dim3 grid(bx, (unsigned)(max_S + 1), (unsigned)n_inst), block(256, 1, 1);
-    hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts, lay, max_L, tile_rows, what);
+    if (what & ~GDP_INIT_FILL) hipLaunchKernelGGL(gdp_init_kernel, grid, block, 0, stream, insts, what & ~GDP_INIT_FILL);
+    if (what & GDP_INIT_FILL) {  // after the poison, if both are asked for
+        if (max_L < 1 || max_L > 65535) return hipErrorInvalidValue;
+        if (bx > 64u) bx = 64u;
+        const int per = 65535 / max_L;  // instances per launch: grid.z holds at most 65535 (instance, layer) pairs
+        for (int i0 = 0; i0 < n_inst; i0 += per) {
+            const int n = n_inst - i0 < per ? n_inst - i0 : per;
+            hipLaunchKernelGGL(gdp_fill_kernel, dim3(bx, (unsigned)max_S, (unsigned)(n * max_L)), block, 0, stream,
+                               insts + i0, lay + (int64_t)i0 * max_L, max_L, tile_rows);
+        }
+    }
     return hipGetLastError();
 }
 
