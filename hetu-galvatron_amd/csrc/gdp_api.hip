@@ -274,7 +274,8 @@ struct Group {  // instances with the same S, sorted by L descending
     struct Segment { int first, layers; unsigned lds_bytes; };
     std::vector<Segment> segments;  // fused launches: runs of layers with the same active set, or -- chunked --
                                     // runs of at most 65535 entries of the row table
-    bool latency = false;           // per-layer launches use the variant for launches with few waves
+    int latency = 0;                // per-layer launches use the variant for launches with few waves: 0, or the
+                                    // number of waves (1, 2, 4) that share the source strategies of a task
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
     std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
     size_t off_rows = 0;
@@ -381,7 +382,8 @@ struct gdp_plan {
     int occupancy_cap_override = 0; // GALVATRON_DP_OCCUPANCY_CAP=n: n workgroups per CU in fused launches
     int chunk_override = 0;         // GALVATRON_DP_CHUNK=n: n instances at a time in fused launches
     int tile_r_override = 0; // GALVATRON_DP_TILE_R: force the register tile height (tuning aid)
-    int latency_override = -1;  // GALVATRON_DP_LATENCY_VARIANT=0|1: never / wherever it exists (tuning aid)
+    int latency_override = -1;  // GALVATRON_DP_LATENCY_VARIANT=0|1|2|4: never / wherever it exists, sources of a
+                                // task on as many waves as the rule says / on 2 / on 4 (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
 
@@ -539,7 +541,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     if (const char *e = getenv("GALVATRON_DP_POISON")) pl->poison = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_SKIP")) pl->skip = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
-    if (const char *e = getenv("GALVATRON_DP_LATENCY_VARIANT")) pl->latency_override = atoi(e) != 0;
+    if (const char *e = getenv("GALVATRON_DP_LATENCY_VARIANT")) pl->latency_override = std::max(0, atoi(e));
     if (const char *e = getenv("GALVATRON_DP_CHUNK")) pl->chunk_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) {
         pl->no_occupancy_cap = atoi(e) == 0;
@@ -700,11 +702,24 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // with all layers in one launch, or on larger problems, it is the slower one).
     for (Group &g : pl->groups) {
         const GdpVariant &v = GDP_VARIANTS[g.variant];
-        g.latency = !pl->fused && !pl->keep_marks && v.ts == GDP_LAT_TS && v.r == GDP_LAT_R;
-        if (pl->latency_override >= 0) g.latency = g.latency_possible(pl->keep_marks) && pl->latency_override != 0;
-        if (g.latency)
+        bool on = !pl->fused && !pl->keep_marks && v.ts == GDP_LAT_TS && v.r == GDP_LAT_R;
+        if (pl->latency_override >= 0) on = g.latency_possible(pl->keep_marks) && pl->latency_override != 0;
+        g.latency = 0;
+        if (on) {
+            // With many sources and wave slots to spare, the sources of a task are split over 2 or 4 waves:
+            // the chain of dependent steps of a layer gets that much shorter.  Measured per solve, 1 / 2 / 4
+            // waves: S=44 V=8192 L=32 0.317 / 0.242 / 0.250 ms, S=64 V=4096 L=16 0.190 / 0.142 / 0.132,
+            // S=44 V=16384 L=16 0.208 / 0.188 / 0.231; no gain or a loss with few sources (S=22 V=16384 L=24
+            // 0.180 / 0.196 / 0.188) or once the waves pass three per SIMD (S=40 V=29493 L=28 0.321 / 0.319 /
+            // 0.388, S=64 V=16384 L=16 0.253 / 0.260 / 0.276).
+            int64_t tasks = 0;
+            for (int k = g.first; k < g.first + g.count; ++k) tasks += (int64_t)inst[(size_t)k].ntile * g.ntb;
+            const int64_t room = (int64_t)pl->num_cu * 4 * 3;  // three waves per SIMD
+            g.latency = g.S < 32 ? 1 : tasks * 4 <= room ? 4 : tasks * 2 <= room ? 2 : 1;
+            if (pl->latency_override >= 1) g.latency = pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1;
             for (int k = g.first; k < g.first + g.count; ++k)
-                inst[(size_t)k].SU = (int)align_up((size_t)inst[(size_t)k].S, GDP_SRC_UNROLL_LAT);
+                inst[(size_t)k].SU = (int)align_up((size_t)inst[(size_t)k].S, (size_t)GDP_SRC_UNROLL_LAT * g.latency);
+        }
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
     size_t off = 0;
@@ -1054,7 +1069,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             for (const Group &g : pl->groups) {
                 if (l >= g.max_L) continue;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, g.latency && !pl->keep_marks,
+                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, pl->keep_marks ? 0 : g.latency,
                                          reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
                                          g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
@@ -1107,7 +1122,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
             t->tile_ts = GDP_VARIANTS[g0.variant].ts;
             t->tile_r = GDP_VARIANTS[g0.variant].r;
             t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
-            t->latency_variant = (!pl->fused && g0.latency) ? 1 : 0;
+            t->latency_variant = pl->fused ? 0 : g0.latency;
         }
         t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));

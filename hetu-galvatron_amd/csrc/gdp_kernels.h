@@ -132,9 +132,10 @@ static const GdpVariant GDP_VARIANTS[] = {
 // One relaxation step (layer `layer`) for the first n_inst instances of the table.
 // marks: track and store the argmin table (otherwise costs only).  lay: the group's table of
 // n_inst x max_L records.
-// latency: the variant for launches too small to hide memory latency behind other waves (costs only,
-// tile GDP_LAT_TS x GDP_LAT_R, SU a multiple of GDP_SRC_UNROLL_LAT); see relax_task_lat.
-hipError_t gdp_launch_relax(int variant, bool marks, bool latency, const GdpDevLayer *lay, int max_L, int n_inst,
+// latency: 0, or K = 1, 2, 4: the variant for launches too small to hide memory latency behind other
+// waves (costs only, tile GDP_LAT_TS x GDP_LAT_R), the source strategies of a task split over K
+// waves; SU is a multiple of K * GDP_SRC_UNROLL_LAT then.  See relax_task_lat.
+hipError_t gdp_launch_relax(int variant, bool marks, int latency, const GdpDevLayer *lay, int max_L, int n_inst,
                             int max_ntile, int SP, int layer, hipStream_t stream);
 #define GDP_LAT_TS 8
 #define GDP_LAT_R 1

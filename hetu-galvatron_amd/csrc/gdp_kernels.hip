@@ -103,17 +103,25 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
 //     step; instruction issue is not what such a launch is short of);
 //   - the row offsets of a whole trip are fetched with the previous trip's.
 // Same arithmetic in the same order as relax_task, hence the same bits.
-template <int TS, int R, bool PUBLISH>
-__device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
+//
+// K > 1: the source strategies of a task are split over K waves of the workgroup (vtb = target block
+// * K + part; part p takes sources [p * SU / K, (p + 1) * SU / K)), which shortens the chain of
+// dependent steps K times where there are wave slots to spare.  The partial minima meet in LDS; the
+// minimum of the parts is the minimum over all sources exactly (min is associative and commutative),
+// and the wave of part j % K adds intra to column j and stores it.
+template <int TS, int R, bool PUBLISH, int K>
+__device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned tile, unsigned vtb, unsigned lane)
 {
     constexpr int NS = 8;
     static_assert(GDP_SRC_UNROLL_LAT % NS == 0 && GDP_SRC_PAD >= 2 * NS, "padding of roff / inter");
-    const int SU = uload(&Y->SU);   // a multiple of NS in the groups this variant runs for
+    static_assert(K == 1 || (R == 1 && GDP_WAVES_PER_BLOCK % K == 0), "parts of one task share a workgroup");
+    const unsigned tb = vtb / K, part = vtb % K;
+    const int SU = uload(&Y->SU) / K;   // a multiple of NS in the groups this variant runs for
     const int SP = uload(&Y->SP);
     const double *src = uload(&Y->src);
-    const int64_t *ro = uload(&Y->ro);
+    const int64_t *ro = uload(&Y->ro) + part * SU;
     const int s0 = tb * TS;
-    const double *it = uload(&Y->it) + s0;
+    const double *it = uload(&Y->it) + s0 + (int64_t)part * SU * SP;
     const int64_t u0 = (int64_t)tile * (64 * R);
     const unsigned lane_bytes = lane * 8u;
     const unsigned col_bytes = (lane < (unsigned)TS ? lane : (unsigned)(TS - 1)) * 8u;
@@ -191,6 +199,25 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
         rop += NS;
     }
 
+    bool mine[TS];
+#pragma unroll
+    for (int j = 0; j < TS; ++j) mine[j] = true;
+    if constexpr (K > 1) {
+        __shared__ double xch[GDP_WAVES_PER_BLOCK][TS][64];
+        const unsigned wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int j = 0; j < TS; ++j) xch[wv][j][lane] = best[0][j];
+        __syncthreads();   // waves of the workgroup that had no task have ended and are not waited for
+        const unsigned w0 = wv - part;   // the task's first wave
+#pragma unroll
+        for (int j = 0; j < TS; ++j) {
+            mine[j] = (unsigned)(j % K) == part;
+            if (mine[j]) {
+#pragma unroll
+                for (int pp = 0; pp < K; ++pp) best[0][j] = min_f64(best[0][j], xch[w0 + pp][j][lane]);
+            }
+        }
+    }
     const GdpDevLayer *Z = Y;
     asm volatile("" : "+s"(Z));
     {
@@ -210,6 +237,7 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
         if (j < nvalid) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
+                if (!mine[j]) continue;
                 if (PUBLISH)
                     __hip_atomic_store(drow + (lane + 64u * r), best[r][j], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
@@ -422,7 +450,8 @@ __device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, 
 // ---- one launch per layer ------------------------------------------------------------------------
 // __launch_bounds__: register allocation is held to 16 resident waves per CU (4 per SIMD, at most
 // 128 VGPRs).
-template <int TS, int R, bool ARG, bool LAT = false>
+// LAT: 0 = the ordinary task; K >= 1: the latency variant with the sources split over K waves.
+template <int TS, int R, bool ARG, int LAT = 0>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_kernel(
     const GdpDevLayer *__restrict__ lay, int max_L, int layer, unsigned ntb)
 {
@@ -440,8 +469,8 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         if (task >= live_tasks) return;
         const unsigned t = task / ntb;
-        if constexpr (LAT)
-            relax_task_lat<TS, R, false>(Y, (unsigned)lo + t, task - t * ntb, lane);
+        if constexpr (LAT > 0)
+            relax_task_lat<TS, R, false, LAT>(Y, (unsigned)lo + t, task - t * ntb, lane);
         else
             relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
     } else if constexpr (ARG) {  // (costs only: those rows were filled when the plan was made)
@@ -899,11 +928,11 @@ __global__ __launch_bounds__(256) void gdp_export_mark_kernel(const GdpDevInst *
 
 }  // namespace
 
-template <int TS, int R, bool ARG, bool LAT = false>
+template <int TS, int R, bool ARG, int LAT = 0>
 static hipError_t launch_relax_t(const GdpDevLayer *lay, int max_L, int n_inst, int max_ntile_rows, int SP, int layer,
                                  hipStream_t stream)
 {
-    const unsigned ntb = (unsigned)(SP / TS);
+    const unsigned ntb = (unsigned)(SP / TS) * (LAT > 1 ? (unsigned)LAT : 1u);  // with the parts of a split task
     const unsigned tasks = (unsigned)max_ntile_rows * ntb;
     unsigned nblk = (tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
     nblk = ((nblk + 7u) & ~7u) + 8u;  // live blocks are rounded up to 8, the fill blocks come after them
@@ -948,14 +977,19 @@ static hipError_t launch_fused_v(bool marks, dim3 grid, dim3 block, unsigned lds
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_relax(int variant, bool marks, bool latency, const GdpDevLayer *lay, int max_L, int n_inst,
+hipError_t gdp_launch_relax(int variant, bool marks, int latency, const GdpDevLayer *lay, int max_L, int n_inst,
                             int max_ntile, int SP, int layer, hipStream_t stream)
 {
     if (latency) {
         if (marks || variant < 0 || variant >= GDP_NUM_VARIANTS || GDP_VARIANTS[variant].ts != GDP_LAT_TS ||
             GDP_VARIANTS[variant].r != GDP_LAT_R)
             return hipErrorInvalidValue;
-        return launch_relax_t<GDP_LAT_TS, GDP_LAT_R, false, true>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+        switch (latency) {
+            case 1: return launch_relax_t<GDP_LAT_TS, GDP_LAT_R, false, 1>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+            case 2: return launch_relax_t<GDP_LAT_TS, GDP_LAT_R, false, 2>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+            case 4: return launch_relax_t<GDP_LAT_TS, GDP_LAT_R, false, 4>(lay, max_L, n_inst, max_ntile, SP, layer, stream);
+            default: return hipErrorInvalidValue;
+        }
     }
 #define X(id, ts, r, m) \
     case id: return launch_relax_v<ts, r, m>(marks, lay, max_L, n_inst, max_ntile, SP, layer, stream);

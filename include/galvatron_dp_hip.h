@@ -103,7 +103,8 @@ typedef struct gdp_timing {
     int32_t tile_r;        /* budget rows per lane                                              */
     int32_t keep_marks;    /* 1: the argmin table is stored while relaxing                      */
     int32_t chunk;         /* instances taken through a fused launch together; 0: all, layer by layer */
-    int32_t latency_variant; /* 1: per-layer launches use the kernel variant for launches with few waves */
+    int32_t latency_variant; /* > 0: per-layer launches use the kernel variant for launches with few waves,
+                                with the source strategies of a task on this many waves (1, 2 or 4) */
     int32_t reserved;
 } gdp_timing;
 

@@ -165,8 +165,9 @@ def test_streams_and_result_buffers_handed_from_plan_to_plan(golden):
 def test_small_launches_use_the_latency_variant(S, monkeypatch):
     """One small instance, one launch per layer: the narrowest tile runs in the variant that keeps
     scalar loads out of its loop (sources padded to 8 per trip, transition costs spread from a vector
-    register).  Same bits as the ordinary variant and as the oracle, f included; S on both sides of
-    the trip length and of the tile width."""
+    register), the sources of a task on 1, 2 or 4 waves whose partial minima meet in LDS.  Same bits
+    as the ordinary variant and as the oracle, f included; S on both sides of the trip length and of
+    the tile width."""
     if any(k in os.environ for k in ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R",
                                      "GALVATRON_DP_FUSED", "GALVATRON_DP_LATENCY_VARIANT")):
         pytest.skip("the environment presets the layout")
@@ -176,7 +177,7 @@ def test_small_launches_use_the_latency_variant(S, monkeypatch):
     wt, wr, wm, wf, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
     keys = sorted(inst.other_mem)
     seen = []
-    for preset in (None, "0"):
+    for preset in (None, "0", "1", "2", "4"):
         if preset is not None:
             monkeypatch.setenv("GALVATRON_DP_LATENCY_VARIANT", preset)
         prob = _problem(inst, export_f=True)
@@ -189,7 +190,8 @@ def test_small_launches_use_the_latency_variant(S, monkeypatch):
                {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
         H.assert_same_results(got, (wt, wr, wm), f"S={S} preset={preset}")
         assert prob.f_out.tobytes() == wf.tobytes()
-    assert seen == [(0, 8, 1, 1), (0, 8, 1, 0)]
+    assert seen[0] == (0, 8, 1, 4 if S >= 32 else 1)        # 12..13 tiles: room for four waves per task
+    assert seen[1:] == [(0, 8, 1, 0), (0, 8, 1, 1), (0, 8, 1, 2), (0, 8, 1, 4)]
 
 
 def test_fused_runs_from_several_threads_take_turns(golden):
