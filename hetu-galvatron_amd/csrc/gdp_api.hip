@@ -370,7 +370,8 @@ struct gdp_plan {
     bool fused = true;            // one launch for all layers instead of one per layer
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
-    int64_t spin_limit = 1 << 22; // polls a waiting wave makes before the launch is abandoned
+    int64_t spin_limit = 1 << 18; // polls a waiting wave makes before the launch is abandoned: about a second
+                                  // (3.5 us apart), a thousand times the longest wait of a healthy launch
     size_t off_zero = 0, zero_words = 0, off_abort = 0;
     int num_cu = 0;
     size_t lds_per_cu = 0;
