@@ -5,33 +5,44 @@
 // allocations below, which is behind a mutex.
 #include "../../include/galvatron_dp_hip.h"
 #include "gdp_kernels.h"
+#include "gdp_host.h"
 
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <condition_variable>
 #include <mutex>
 #include <new>
 #include <string>
 #include <vector>
 
+// ---- shared with gdp_static.hip (declared in gdp_host.h) ---------------------------------------------
 namespace {
+thread_local char g_err[320] = "";   // a fixed buffer: reporting an error allocates nothing
+}
 
-thread_local std::string g_err;
+void gdp_clear_error() { g_err[0] = 0; }
 
-int fail(int code, const std::string &msg)
+int gdp_fail(int code, const char *msg)
 {
-    g_err = msg;
+    snprintf(g_err, sizeof g_err, "%s", msg ? msg : "");
     return code;
 }
 
-int fail_hip(hipError_t e, const char *what)
+int gdp_fail_hip(hipError_t e, const char *what)
 {
     // a failed allocation is reported as such; everything else as a runtime error
     const int code = (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) ? GDP_E_NOMEM : GDP_E_HIP;
-    return fail(code, std::string(what) + ": " + hipGetErrorString(e));
+    snprintf(g_err, sizeof g_err, "%s: %s", what, hipGetErrorString(e));
+    return code;
 }
+
+namespace {
+
+int fail(int code, const char *msg) { return gdp_fail(code, msg); }
+int fail_hip(hipError_t e, const char *what) { return gdp_fail_hip(e, what); }
 
 #define GDP_HIP(call)                                    \
     do {                                                 \
@@ -45,7 +56,7 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Getting fresh device memory costs far more than filling it (94 GB for 256 Llama-7B-like instances:
 // 2.7 s to allocate, 0.05 s to solve), and the search engine solves thousands of DPs in a row.  The
 // allocation of a finished plan is therefore kept for the next plan on that device instead of being
-// freed: up to GALVATRON_DP_CACHE_MB (default 20480, 0 = keep nothing) in total -- room for the two
+// freed: up to GALVATRON_DP_CACHE_MB (default 20480 or an eighth of the device memory, whichever is less; 0 = keep nothing) in total -- room for the two
 // allocations of GALVATRON_DP_ARENA_MB that a batch solved in parts works in, and the small ones of
 // single solves between such batches --, the ones given back longest ago given up first when that is
 // exceeded, all of them on an out-of-memory error or gdp_cache_trim().
@@ -120,9 +131,32 @@ hipError_t arena_take(int device, size_t need, char **ptr, size_t *bytes)
     return e;
 }
 
+// What may stay cached on `device`: GALVATRON_DP_CACHE_MB if set, else 20 GB but never more than an
+// eighth of the device's memory (a process that shares the device with other work can set it to 0, or
+// call gdp_cache_trim() when its search is over).
+size_t cache_cap(int device)
+{
+    const char *e = getenv("GALVATRON_DP_CACHE_MB");
+    if (e && *e) return env_mb("GALVATRON_DP_CACHE_MB", 0);
+    static std::mutex mu;
+    static std::vector<size_t> total;  // per device, 0 = not asked yet
+    std::lock_guard<std::mutex> lk(mu);
+    if (device >= 0 && (size_t)device >= total.size()) total.resize((size_t)device + 1, 0);
+    if (device >= 0 && total[(size_t)device] == 0) {
+        size_t t = 0;
+        if (hipDeviceTotalMem(&t, device) != hipSuccess || t == 0) {
+            (void)hipGetLastError();
+            t = (size_t)64 << 30;
+        }
+        total[(size_t)device] = t;
+    }
+    const size_t eighth = device >= 0 ? total[(size_t)device] / 8 : (size_t)8 << 30;
+    return std::min((size_t)20480 << 20, eighth);
+}
+
 void arena_give(int device, char *ptr, size_t bytes)
 {
-    const size_t cap = env_mb("GALVATRON_DP_CACHE_MB", 20480);
+    const size_t cap = cache_cap(device);
     std::vector<Arena> drop;
     if (bytes > cap) {
         drop.push_back({device, ptr, bytes});
@@ -251,7 +285,29 @@ void lane_trim()
 // side can fill an XCD each with workgroups waiting for one that needs a place on the other XCD;
 // the bounded wait then runs out (seconds) and both fall back to per-layer launches.  Launches
 // without such waits (one per layer) may run beside a fused one: their workgroups always finish.
+// The turn is a flag under a mutex, not a held mutex: a run may be started by one thread and waited for
+// (or its plan destroyed) by another.  It orders the threads of ONE process; another process on the same
+// device is not seen (its fused launches and these can then block each other until the bounded wait of
+// one of them runs out, after which that plan continues with one launch per layer).
 std::mutex g_fused_mu;
+std::condition_variable g_fused_cv;
+bool g_fused_busy = false;
+
+void fused_turn_take()
+{
+    std::unique_lock<std::mutex> lk(g_fused_mu);
+    g_fused_cv.wait(lk, [] { return !g_fused_busy; });
+    g_fused_busy = true;
+}
+
+void fused_turn_give()
+{
+    {
+        std::lock_guard<std::mutex> lk(g_fused_mu);
+        g_fused_busy = false;
+    }
+    g_fused_cv.notify_one();
+}
 
 struct HostInst {
     int orig;  // index in the caller's arrays
@@ -330,13 +386,17 @@ int pick_ts(int S, bool marks, int64_t tiles, int64_t wave_slots)
 
 int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
 
-int find_variant(int ts, int r)
+}  // namespace
+
+int gdp_find_variant(int ts, int r)
 {
     for (int v = 0; v < GDP_NUM_VARIANTS; ++v)
         if (GDP_VARIANTS[v].ts == ts && GDP_VARIANTS[v].r == r) return v;
     return -1;
 }
 
+namespace {
+int find_variant(int ts, int r) { return gdp_find_variant(ts, r); }
 }  // namespace
 
 struct gdp_plan {
@@ -366,7 +426,7 @@ struct gdp_plan {
     double executed = 0;     // relaxations actually carried out (tiles inside the bands)
     bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
     bool ran = false;
-    bool holds_fused = false;     // between run_enqueue and run_finish of a fused run: g_fused_mu is held
+    bool holds_fused = false;     // between run_enqueue and run_finish of a fused run: this plan has the turn
     bool fused = true;            // one launch for all layers instead of one per layer
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
@@ -388,9 +448,7 @@ struct gdp_plan {
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
 };
 
-namespace {
-
-int validate(const gdp_problem *p, int i)
+int gdp_validate(const gdp_problem *p, int i)
 {
     char buf[160];
     auto bad = [&](int code, const char *why) {
@@ -399,6 +457,8 @@ int validate(const gdp_problem *p, int i)
     };
     if (!p) return bad(GDP_E_BADARG, "null problem");
     if (p->L < 1 || p->V < 1 || p->S < 1) return bad(GDP_E_BADARG, "L, V and S must be >= 1");
+    if (p->V > GDP_MAX_V) return bad(GDP_E_BADARG, "V exceeds GDP_MAX_V");
+    if (p->L > GDP_MAX_L) return bad(GDP_E_BADARG, "L exceeds GDP_MAX_L");
     if (p->S > GDP_MAX_S) return bad(GDP_E_BADARG, "S exceeds GDP_MAX_S");
     if (p->S > GDP_MAX_S_MARKS && (p->flags & (GDP_KEEP_MARKS | GDP_EXPORT_MARK)))
         return bad(GDP_E_BADARG, "S exceeds GDP_MAX_S_MARKS and the argmin table was asked for");
@@ -428,36 +488,60 @@ int validate(const gdp_problem *p, int i)
         }
         bound += m;
     }
-    std::vector<double> tmax((size_t)T, 0.0);
+    // This function allocates nothing: the per-matrix maxima live in a small fixed table, and with more
+    // matrices than that a matrix shared by several layers is simply scanned once per layer.
     const size_t SS = (size_t)p->S * p->S;
-    for (int t = 0; t < T; ++t) {
+    auto matrix_max = [&](int t, double *m_out) {
         double m = 0;
         const double *q = p->inter + (size_t)t * SS;
         for (size_t k = 0; k < SS; ++k) {
             const double x = q[k];
-            if (x != x || x == -INFINITY) return bad(GDP_E_NONFINITE, "NaN or -inf in inter");
+            if (x != x || x == -INFINITY) return false;
             if (x != INFINITY) m = std::max(m, std::fabs(x));
         }
-        tmax[t] = m;
+        *m_out = m;
+        return true;
+    };
+    constexpr int TMAX_KEPT = 64;
+    double tmax[TMAX_KEPT];
+    const bool kept = p->inter_index && T <= TMAX_KEPT;
+    if (p->inter_index)  // every matrix is checked, also one that no layer uses
+        for (int t = 0; t < T; ++t) {
+            double m = 0;
+            if (!matrix_max(t, &m)) return bad(GDP_E_NONFINITE, "NaN or -inf in inter");
+            if (kept) tmax[t] = m;
+        }
+    for (int l = 0; l < p->L; ++l) {
+        double m = 0;
+        if (kept) m = tmax[p->inter_index[l]];
+        else if (!matrix_max(p->inter_index ? p->inter_index[l] : l, &m))
+            return bad(GDP_E_NONFINITE, "NaN or -inf in inter");
+        bound += m;
     }
-    for (int l = 0; l < p->L; ++l) bound += tmax[p->inter_index ? p->inter_index[l] : l];
     for (int k = 0; k < p->n_key; ++k) {
         const double x = p->other_time[k];
         if (x != x || x == -INFINITY) return bad(GDP_E_NONFINITE, "NaN or -inf in other_time");
+        // start row V-1-other_mem (csrc/dp_core.cpp:82): a negative entry puts it above the table, where the
+        // reference reads out of bounds; an entry above V-1 is an infeasible key and is answered as such
+        if (p->other_mem[k] < 0) return bad(GDP_E_BADARG, "negative other_mem entry (start row above the table)");
     }
     if (!(bound < 1e300)) return bad(GDP_E_NONFINITE, "cost magnitudes could overflow binary64");
     return GDP_OK;
 }
 
+namespace {
+
+int validate(const gdp_problem *p, int i) { return gdp_validate(p, i); }
+
 void destroy(gdp_plan *pl)
 {
     if (!pl) return;
-    if (pl->holds_fused) {  // a run that was started and never waited for
-        pl->holds_fused = false;
-        g_fused_mu.unlock();
-    }
     if (pl->dbase || pl->lane.stream) (void)hipSetDevice(pl->device);
     if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read its host copy
+    if (pl->holds_fused) {  // a run that was started and never waited for: its launch has ended by now
+        pl->holds_fused = false;
+        fused_turn_give();
+    }
     if (pl->dbase) arena_give(pl->device, pl->dbase, pl->dalloc);
     for (hipEvent_t e : pl->ev_relax) (void)hipEventDestroy(e);
     lane_give(pl->lane);
@@ -731,6 +815,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     };
     int nk = 0;
     size_t nres = 0;
+    {
+        // the key table and the array of strategy lists are indexed with 32-bit offsets on the device
+        size_t keys = 0, lists = 0;
+        for (const auto &h : inst) {
+            keys += (size_t)h.n_key;
+            lists += (size_t)h.n_key * (size_t)h.L;
+        }
+        if (keys > (size_t)INT32_MAX || lists > (size_t)INT32_MAX)
+            return fail(GDP_E_BADARG, "more than 2^31-1 keys or strategy-list entries in one plan");
+    }
     for (auto &h : inst) {
         h.key_begin = nk; nk += h.n_key;
         h.res_begin = (int)nres; nres += (size_t)h.n_key * h.L;
@@ -1049,7 +1143,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     }
     size_t li = 0;
     if (pl->fused && !pl->holds_fused) {
-        g_fused_mu.lock();  // until run_finish has waited for the launch (same thread)
+        fused_turn_take();  // until run_finish has waited for the launch
         pl->holds_fused = true;
     }
     if (pl->fused) {
@@ -1093,7 +1187,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
     const hipError_t waited = hipStreamSynchronize(pl->stream);
     if (pl->holds_fused) {
         pl->holds_fused = false;
-        g_fused_mu.unlock();
+        fused_turn_give();
     }
     GDP_HIP(waited);
     pl->h_out = reinterpret_cast<const GdpDevOut *>(pl->lane.back + (pl->off_out - pl->off_abort));
@@ -1144,8 +1238,9 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t)
 {
     const int rc = run_enqueue(pl, mode);
     if (rc != GDP_OK && pl->holds_fused) {  // a launch failed: nothing to wait for
+        (void)hipStreamSynchronize(pl->stream);
         pl->holds_fused = false;
-        g_fused_mu.unlock();
+        fused_turn_give();
     }
     return rc == GDP_OK ? run_finish(pl, mode, t) : rc;
 }
@@ -1198,14 +1293,6 @@ int fetch(gdp_plan *pl, gdp_result *const *r)
     return GDP_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-}  // extern "C"
-
-namespace {
-
 // A plan for problems that validate() has accepted.
 int create_checked(int32_t n, const gdp_problem *const *p, gdp_plan **out)
 {
@@ -1235,7 +1322,7 @@ extern "C" {
 
 int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!out) return fail(GDP_E_BADARG, "null plan pointer");
     *out = nullptr;
     if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
@@ -1249,21 +1336,21 @@ int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
 
 int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!plan) return fail(GDP_E_BADARG, "null plan");
     return run(plan, timing ? timing_mode : 0, timing);
 }
 
 int gdp_plan_fetch(gdp_plan *plan, gdp_result *const *r)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!plan || !r) return fail(GDP_E_BADARG, "null plan or results");
     return fetch(plan, r);
 }
 
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!plan) return fail(GDP_E_BADARG, "null plan");
     switch (option) {
         case GDP_OPT_FUSED:
@@ -1299,7 +1386,7 @@ void gdp_cache_trim(void)
 
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!r) return fail(GDP_E_BADARG, "null results");
     if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
     for (int i = 0; i < n; ++i) {  // all of them first: nothing is written when one is rejected
@@ -1330,8 +1417,9 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
         if (rc == GDP_OK && rp == GDP_OK) {
             rc = run_enqueue(pl, 0);
             if (rc != GDP_OK && pl->holds_fused) {
+                (void)hipStreamSynchronize(pl->stream);
                 pl->holds_fused = false;
-                g_fused_mu.unlock();
+                fused_turn_give();
             }
         }
         if (prev) {
@@ -1361,13 +1449,13 @@ int gdp_solve(const gdp_problem *p, gdp_result *r)
     return gdp_solve_batch(1, pp, rr);
 }
 
-const char *gdp_last_error(void) { return g_err.c_str(); }
+const char *gdp_last_error(void) { return g_err; }
 
 int gdp_version(void) { return GDP_VERSION; }
 
 int gdp_device_info(char *buf, size_t len)
 {
-    g_err.clear();
+    gdp_clear_error();
     if (!buf || len == 0) return fail(GDP_E_BADARG, "null buffer");
     int dev = 0;
     GDP_HIP(hipGetDevice(&dev));

@@ -34,13 +34,15 @@ extern "C" {
 
 /* return codes */
 #define GDP_OK 0
-#define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S above GDP_MAX_S(_MARKS), ... */
+#define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S / V / L above GDP_MAX_*, negative mem or other_mem, ... */
 #define GDP_E_UNSUPPORTED (-2) /* an input the device recurrence does not cover: mem <= 0 */
 #define GDP_E_NONFINITE (-3)   /* NaN or -inf in a cost array (the reference's result is then order-dependent) */
 #define GDP_E_NOMEM (-4)       /* device or host allocation failed */
 #define GDP_E_HIP (-5)         /* any other HIP runtime error; text in gdp_last_error() */
 
 #define GDP_MAX_S 1024      /* strategies per layer */
+#define GDP_MAX_V (1 << 30) /* budget bins */
+#define GDP_MAX_L 65535     /* layers */
 #define GDP_MAX_S_MARKS 256 /* ... when the argmin table is kept (GDP_KEEP_MARKS, GDP_EXPORT_MARK): its entries are bytes */
 
 /* gdp_problem.flags */
@@ -70,7 +72,8 @@ typedef struct gdp_problem {
     const int32_t *inter_index; /* [L] layer -> matrix in `inter`; NULL means n_inter == L, identity */
     int32_t n_inter;
     int32_t n_key;              /* number of (other_mem, other_time) pairs to finish for           */
-    const int64_t *other_mem;   /* [n_key]                                                         */
+    const int64_t *other_mem;   /* [n_key]  every entry must be >= 0 (start row V-1-other_mem inside the table;
+                                            an entry above V-1 is an infeasible key: total +inf, remaining -1) */
     const double *other_time;   /* [n_key]                                                         */
     uint32_t flags;
 } gdp_problem;
@@ -149,7 +152,7 @@ void gdp_plan_destroy(gdp_plan *plan);
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
 
 /* Frees the device allocations that finished plans left behind for reuse (no counterpart in the
- * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 20480, 0 keeps
+ * reference).  The library keeps them, up to GALVATRON_DP_CACHE_MB in total (default 20480 or an eighth of the device memory, whichever is less; 0 keeps
  * nothing), because obtaining device memory costs far more than a solve.  Finished plans also leave
  * their stream, two events and page-locked result buffer for the next plan (at most 64 sets; creating
  * and destroying a stream takes a third as long as a small solve); this call releases those too. */

@@ -66,6 +66,14 @@ def test_validation_happens_before_any_device_work():
     p = _lib.Problem(np.ones((1, n), np.int32), np.ones((1, n)), np.zeros((1, n, n)), 10, [0], [0.0], keep_marks=True)
     assert rc_of(p)[0] == _lib.GDP_E_BADARG
     assert lib.gdp_plan_create(0, None, ctypes.byref(ctypes.c_void_p())) == _lib.GDP_E_BADARG
+    # a negative other_mem would put the start row V-1-other_mem above the table (the reference reads out of
+    # bounds there, csrc/dp_core.cpp:82-89); one above V-1 is merely an infeasible key and is accepted
+    rc, msg = rc_of(_lib.Problem(mem, intra, inter, 10, [0, -1], [0.0, 0.0]))
+    assert rc == _lib.GDP_E_BADARG and "other_mem" in msg
+    rc, msg = rc_of(_lib.Problem(mem, intra, inter, 10, [-(1 << 40)], [0.0]))
+    assert rc == _lib.GDP_E_BADARG and "other_mem" in msg
+    too_tall = _lib.Problem(mem, intra, inter, (1 << 30) + 1, [0], [0.0])
+    assert rc_of(too_tall)[0] == _lib.GDP_E_BADARG
 
 
 def test_problem_shape_checks():
