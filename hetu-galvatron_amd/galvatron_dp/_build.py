@@ -12,7 +12,7 @@ PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libgalvatron_dp_hip.so")
-SOURCES = ["gdp_kernels.hip", "gdp_api.hip"]
+SOURCES = ["gdp_kernels.hip", "gdp_api.hip", "gdp_static.hip"]
 ARCH = "gfx950"
 # -ffp-contract=off: the recurrence has no multiply, but nothing may ever be fused or reassociated.
 # packed-fp32-ops is switched off for every HIP translation unit built here.

@@ -34,7 +34,9 @@ GDP_OPT_SPIN_LIMIT = 2
 GDP_OPT_POISON = 3
 GDP_OPT_NO_FALLBACK = 4
 
-EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
+GDP_STATIC_SCRATCH_BYTES = 64 << 20
+
+EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_solve_static", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
                     "gdp_plan_destroy", "gdp_plan_set_option", "gdp_cache_trim", "gdp_last_error", "gdp_version",
                     "gdp_device_info")
 
@@ -80,6 +82,8 @@ def lib() -> ctypes.CDLL:
         rp = ctypes.POINTER(ctypes.POINTER(gdp_result))
         L.gdp_solve.argtypes = [ctypes.POINTER(gdp_problem), ctypes.POINTER(gdp_result)]
         L.gdp_solve.restype = ctypes.c_int
+        L.gdp_solve_static.argtypes = [ctypes.POINTER(gdp_problem), ctypes.POINTER(gdp_result)]
+        L.gdp_solve_static.restype = ctypes.c_int
         L.gdp_solve_batch.argtypes = [ctypes.c_int32, pp, rp]
         L.gdp_solve_batch.restype = ctypes.c_int
         L.gdp_plan_create.argtypes = [ctypes.c_int32, pp, ctypes.POINTER(ctypes.c_void_p)]
@@ -202,6 +206,11 @@ def solve_batch(problems: Sequence[Problem]) -> None:
         return
     P, R = _arrays(problems)
     _check(lib().gdp_solve_batch(len(problems), P, R))
+
+
+def solve_static(problem: Problem) -> None:
+    """gdp_solve_static: one instance, solved in the library's static device array (no allocation)."""
+    _check(lib().gdp_solve_static(ctypes.byref(problem._c_problem), ctypes.byref(problem._c_result)))
 
 
 class Plan:

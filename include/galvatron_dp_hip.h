@@ -124,6 +124,25 @@ int gdp_solve(const gdp_problem *p, gdp_result *r);
  * reuse one allocation. */
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r);
 
+/* gdp_solve for callers that cannot allocate.  No counterpart in the reference: it exists for callers that
+ * may not obtain memory while they run -- code executing while a HIP graph is being captured, serving
+ * loops that must stay off the allocator, harnesses that forbid hipMalloc.  Same arguments (host
+ * pointers, borrowed for the call) and the same results, bit for bit, as gdp_solve, but the call
+ * obtains no device memory, no page-locked memory, no stream and no event, and uses no host allocator:
+ * its cost buffers, argmin table, tables and results live in one static device array of
+ * GDP_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends, the
+ * inputs' device layout is built in a fixed host array, and the work runs on the null stream with
+ * synchronous copies.  It keeps two cost buffers and the one-byte argmin table (the layout of
+ * GDP_KEEP_MARKS), one launch per layer, every cell computed.
+ *   - An instance that needs more than the array (roughly 17*(V + max mem)*(S+1) + L*S*V bytes, or
+ *     tables above 8 MiB) is refused with GDP_E_NOMEM and a message that gives both sizes; so are
+ *     S > GDP_MAX_S_MARKS and the export flags (GDP_E_BADARG).  Other flags are ignored.
+ *   - All calls of a process share the array of their device, which keeps what the last call left; a
+ *     call rewrites everything it reads, and calls take a process-wide lock, so they run one after the
+ *     other.  Work that other code queues on the null stream is ordered with it as usual. */
+#define GDP_STATIC_SCRATCH_BYTES (64 << 20)
+int gdp_solve_static(const gdp_problem *p, gdp_result *r);
+
 /* The same in three steps, so that a caller (or a benchmark) can keep inputs resident in
  * device memory and run the device part repeatedly:
  *   create  -- validate + allocate + copy inputs to the device

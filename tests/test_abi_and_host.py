@@ -76,6 +76,26 @@ def test_validation_happens_before_any_device_work():
     assert rc_of(too_tall)[0] == _lib.GDP_E_BADARG
 
 
+def test_static_entry_point_refuses_on_the_host():
+    """gdp_solve_static checks the arguments and the size of its fixed working memory before it touches
+    the device: an instance that does not fit is refused with both sizes in the message."""
+    lib = _lib.lib()
+    S, L, V = 44, 32, 65536                          # the argmin table alone is 92 MB
+    p = _lib.Problem(np.ones((L, S), np.int32), np.ones((L, S)), np.zeros((1, S, S)), V, [0], [0.0],
+                     inter_index=np.zeros(L, np.int32))
+    rc = lib.gdp_solve_static(ctypes.byref(p._c_problem), ctypes.byref(p._c_result))
+    msg = lib.gdp_last_error().decode()
+    assert rc == _lib.GDP_E_NOMEM and str(_lib.GDP_STATIC_SCRATCH_BYTES) in msg and "gdp_solve" in msg, msg
+    with pytest.raises(MemoryError):
+        _lib.solve_static(p)
+    mem = np.ones((2, 3), np.int32)
+    q = _lib.Problem(mem, np.ones((2, 3)), np.zeros((2, 3, 3)), 10, [0], [0.0], export_f=True)
+    assert lib.gdp_solve_static(ctypes.byref(q._c_problem), ctypes.byref(q._c_result)) == _lib.GDP_E_BADARG
+    q = _lib.Problem(mem, np.ones((2, 3)), np.zeros((2, 3, 3)), 10, [-2], [0.0])
+    assert lib.gdp_solve_static(ctypes.byref(q._c_problem), ctypes.byref(q._c_result)) == _lib.GDP_E_BADARG
+    assert lib.gdp_solve_static(None, None) == _lib.GDP_E_BADARG
+
+
 def test_problem_shape_checks():
     with pytest.raises(ValueError):
         _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 4)), np.zeros((2, 3, 3)), 10, [0], [0.0])
