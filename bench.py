@@ -12,16 +12,27 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    both sides).  The timed solves carry out EVERY one of the L*V*S*S relaxations
                    (GDP_COMPUTE_ALL); ``with_row_skipping`` reports the library's default, which
                    skips rows it can prove irrelevant and returns identical results.
-* ``roofline``     for the relaxation kernel (the only kernel that matters): the ALGORITHMIC 3 fp64
-                   vector operations per relaxation (two additions and one comparison per candidate,
-                   as the reference's loop does them), divided by the average launch duration
-                   measured with HIP events on the stream the kernel runs on;
-                   peak = 39.3 TFLOP/s = MI355X's published 78.6 TFLOP/s fp64 vector rate, which
-                   counts an FMA as two operations -- additions and comparisons cannot fuse.
-                   The kernel itself issues fewer: one addition and one minimum per relaxation plus
-                   one addition per cell (intra is added after the minimum, which is exact because
-                   rounding is monotone); ``issued_ops_per_relaxation`` and ``frac_issued`` give the
-                   fraction of the peak in instructions actually issued.
+* ``roofline``     for the relaxation kernel (the only kernel that matters): the fp64 vector
+                   operations the kernel needs AND ISSUES for the relaxations it carries out -- one
+                   addition and one minimum per relaxation plus one addition per cell, 2 + 1/S (intra
+                   is added after the minimum, which is exact because rounding is monotone); five per
+                   relaxation where the argmin table is stored, four + 1/S in the variant for small
+                   launches -- divided by the average launch duration measured with HIP events on the
+                   stream the kernel runs on; peak = 39.3 T operations/s = MI355X's published
+                   78.6 TFLOP/s fp64 vector rate, which counts an FMA as two operations (additions and
+                   minima cannot fuse) at the published 2.4 GHz.  ``frac`` is therefore a fraction of
+                   the instruction-issue roof and cannot exceed 1.  ``frac_reference_ops`` counts the 3
+                   operations per relaxation of the reference's loop body (two additions and one
+                   comparison, csrc/dp_core.cpp:65-73) over the same time: it can exceed 1, because the
+                   kernel does not execute that work.  ``clock_ghz_under_load`` is the shader clock
+                   read from sysfs while the timed steps ran (null where the file is not readable;
+                   the SQ cycle counters in profiles/ give 2.05-2.10 GHz for cfg2).
+                   ``traffic`` is the measured HBM-side byte count per launch from profiles/, given
+                   only while the kernel sources still hash to what was profiled.
+* ``vs_baseline``  null: the reference publishes no number for this path.
+* ``also``         the other workloads, shorter legs, each with its own fractions and a ``bit_exact``
+                   flag: results compared, outside the timed region, with the committed vectors
+                   written from the reference's compiled dp_core (tests/golden/dp_core_golden.json).
                    ``roofline_hbm`` is the same launch against 8 TB/s with the algorithmic bytes
                    V*S*(8 read + 8 write) per layer and instance (the relaxation stores costs only;
                    the backtrack recomputes the argmin of the L cells on its path.  ``with_mark_table``
@@ -52,12 +63,102 @@ PEAK_FP64_VALU_TFLOPS = 39.3   # 78.6 TFLOP/s published (FMA = 2 ops) / 2
 PEAK_HBM_GBS = 8000.0
 # Bytes per launch of the relaxation kernel between the L2s and the fabric (HBM and the memory-side
 # cache in front of it), measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a copy
-# kernel of known size; see profiles/.  None where not measured.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "cfg2": 12.131e9,   # profiles/gdp_relax_fused_kernel_cfg2.txt  (algorithmic 10.737e9; one launch per solve)
-    "cfg3": 45.8e9,     # profiles/gdp_relax_fused_kernel_cfg3.txt  (algorithmic 44.3e9; average of the 4 launches of a solve)
-    "cfg2+row_skipping": 7.652e9,   # profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt
+# kernel of known size; see profiles/.  Each figure belongs to the kernel sources it was measured on
+# (first 16 hex digits of the SHA-256 of gdp_kernels.hip + gdp_kernels.h) and to one register tile; the
+# bench line carries it only while both still match, null otherwise.
+MEASURED_TRAFFIC = {
+    # workload (+ mode): (bytes per launch, kernel sources hash, register tile "TSxR", profile)
+    "cfg2": (12.131e9, "", "16x1", "profiles/gdp_relax_fused_kernel_cfg2.txt"),
+    "cfg3": (45.8e9, "", "15x1", "profiles/gdp_relax_fused_kernel_cfg3.txt"),
+    "cfg2+row_skipping": (7.652e9, "", "16x1", "profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt"),
 }
+KERNEL_SOURCES = ("hetu-galvatron_amd/csrc/gdp_kernels.hip", "hetu-galvatron_amd/csrc/gdp_kernels.h")
+GOLDEN = os.path.join(ROOT, "tests", "golden", "dp_core_golden.json")
+
+
+def _kernel_sources_hash() -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def _traffic(key: str, tile: str):
+    rec = MEASURED_TRAFFIC.get(key)
+    if rec is None:
+        return None, "not measured for this workload"
+    nbytes, src_hash, rec_tile, profile = rec
+    if src_hash != _kernel_sources_hash() or rec_tile != tile:
+        return None, f"{profile} was measured on other kernel sources or another register tile"
+    return nbytes, profile
+
+
+class _ClockSampler:
+    """Shader clock while the timed steps run: the level marked '*' in the amdgpu sysfs file
+    pp_dpm_sclk, sampled from a thread.  None where no such file is readable."""
+
+    def __init__(self):
+        import glob
+        self.paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.samples = []
+        self._stop = False
+        self._thread = None
+
+    def _read(self):
+        for p in self.paths:
+            try:
+                with open(p) as fh:
+                    for ln in fh:
+                        if "*" in ln:
+                            return float(ln.split(":")[1].strip().split("M")[0]) / 1e3
+            except (OSError, ValueError, IndexError):
+                continue
+        return None
+
+    def __enter__(self):
+        import threading
+        if self.paths:
+            def loop():
+                while not self._stop:
+                    v = self._read()
+                    if v:
+                        self.samples.append(v)
+                    time.sleep(0.002)
+            self._thread = threading.Thread(target=loop, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+
+    def ghz(self):
+        return sorted(self.samples)[len(self.samples) // 2] if self.samples else None
+
+
+def _bit_exact(workload: str, probs) -> bool | None:
+    """Results of the solved problems against the committed vectors written from the reference's
+    compiled dp_core; None when the file or the case is absent."""
+    if not os.path.exists(GOLDEN):
+        return None
+    with open(GOLDEN) as fh:
+        golden = json.load(fh)
+    names = [f"cfg3_{n:03d}" for n in range(len(probs))] if workload == "cfg3" else [workload]
+    import numpy as np
+    for name, prob in zip(names, probs):
+        rec = golden.get(name)
+        if rec is None:
+            return None
+        total = np.array([float.fromhex(h) for h in rec["total_hex"]])
+        if total.tobytes() != prob.total.tobytes() or list(prob.remaining) != list(rec["remaining"]):
+            return False
+        for k, want in enumerate(rec["res"]):
+            if prob.remaining[k] != -1 and [int(x) for x in prob.res[k]] != list(want):
+                return False
+    return True
 
 
 def _problems(workload: str, compute_all: bool = True, keep_marks: bool = False):
@@ -147,7 +248,7 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true",
                     help="leave out the row-skipping and mark-table legs (profiling runs: the trace then holds the "
                          "headline's launches alone)")
-    ap.add_argument("--also", default="cfg3", help="comma-separated extra workloads summarised in the same line")
+    ap.add_argument("--also", default="cfg3,cfg0,cfg1,cfg4", help="comma-separated extra workloads summarised in the same line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run three device-to-device copies of 1 GiB (a kernel of known traffic, to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
@@ -181,20 +282,29 @@ def main() -> int:
         print(json.dumps({"calibrate_copy_bytes": n, "copies": 3}))
         return 0
 
-    def measure(workload, steps, warmup, compute_all=True, keep_marks=False, host_leg=False):
+    def measure(workload, steps, warmup, compute_all=True, keep_marks=False, host_leg=False, check=False):
         insts, probs = _problems(workload, compute_all, keep_marks)
         with _lib.Plan(probs) as plan:
             for _ in range(warmup):
                 plan.run(0)
             device_sync()
-            t0 = time.perf_counter()
-            for _ in range(steps):
-                plan.run(0)                       # synchronises the plan's stream before returning
-            device_sync()
-            wall = time.perf_counter() - t0
+            with _ClockSampler() as clock:
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    plan.run(0)                       # synchronises the plan's stream before returning
+                device_sync()
+                wall = time.perf_counter() - t0
             tm = plan.run(2)                       # per-launch HIP events on the plan's stream
             t1 = plan.run(1)
             plan.fetch()
+        bit_exact = None
+        if check:                                  # outside the timed region
+            bit_exact = _bit_exact(workload, probs)
+            if bit_exact is not None:
+                with open(GOLDEN) as fh:
+                    golden = json.load(fh)
+                names = [f"cfg3_{n:03d}" for n in range(len(insts))] if workload == "cfg3" else [workload]
+                bit_exact = bit_exact and all(i.digest() == golden[n]["input_sha256"] for i, n in zip(insts, names))
         # The same solve from host arrays through gdp_solve_batch: validation, layout, upload, all kernels,
         # download (device memory of earlier calls is reused).  Reported beside the headline, never as it.
         host_ms = []
@@ -206,26 +316,38 @@ def main() -> int:
         relax = tm.relaxations
         launches = tm.relax_launches
         avg_launch_s = tm.relax_ms * 1e-3 / launches
+        # fp64 vector operations the kernel issues per relaxation: v_add_f64 + v_min_f64, plus one addition
+        # per cell (1/S); with the argmin table two additions, compare, select, minimum; the variant for
+        # small per-layer launches spends two more (v_readlane) on spreading the transition costs
+        issued = 5.0 if keep_marks else (4.0 if tm.latency_variant else 2.0) + 1.0 / insts[0].S
+        per_launch_s = tm.executed / launches / avg_launch_s
         return {
             "insts": insts, "probs": probs, "relaxations": relax, "ms_per_step": wall / steps * 1e3,
             "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
             "device_ms": t1.total_ms, "host_ms": host_ms, "executed_fraction": tm.executed / relax,
-            "tflops": 3.0 * tm.executed / launches / avg_launch_s / 1e12,
-            # the variant for small per-layer launches spends two more vector instructions per relaxation on
-            # spreading the transition costs from a vector register (v_readlane)
-            "issued_per_relaxation": 5.0 if keep_marks else (4.0 if tm.latency_variant else 2.0) + 1.0 / insts[0].S,
+            "tops_issued": issued * per_launch_s / 1e12, "tops_reference": 3.0 * per_launch_s / 1e12,
+            "issued_per_relaxation": issued,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
             "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
             "tile": "%d target strategies x %d budget rows per wavefront" % (tm.tile_ts, 64 * tm.tile_r),
+            "tile_key": "%dx%d" % (tm.tile_ts, tm.tile_r),
             "kernel": "gdp_relax_fused_kernel" if tm.fused else
                       ("gdp_relax_kernel (latency variant)" if tm.latency_variant else "gdp_relax_kernel"),
+            "clock_ghz": clock.ghz(), "bit_exact": bit_exact,
         }
 
-    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping, host_leg=not a.headline_only)
+    def fractions(mm):
+        return {"frac": mm["tops_issued"] / PEAK_FP64_VALU_TFLOPS,
+                "frac_reference_ops": mm["tops_reference"] / PEAK_FP64_VALU_TFLOPS,
+                "frac_hbm": mm["gbs"] / PEAK_HBM_GBS}
+
+    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping, host_leg=not a.headline_only,
+                check=True)
     insts = m["insts"]
     first = insts[0]
-    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(a.workload + ("+row_skipping" if a.row_skipping else ""))
+    traffic, traffic_source = _traffic(a.workload + ("+row_skipping" if a.row_skipping else ""), m["tile_key"])
+    fr = fractions(m)
     line = {
         "metric": "min-plus relaxations/s (L*V*S^2)", "value": m["value"], "unit": "relaxations/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": m["ms_per_step"],
@@ -235,25 +357,31 @@ def main() -> int:
                    "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"],
                    "search_wall_ms_from_host_arrays": m["host_ms"], "launch_scheme": m["scheme"],
                    "register_tile": m["tile"],
-                   "relaxations_executed_fraction": m["executed_fraction"], "device": _lib.device_info()},
-        "roofline": {"bound": "valu_fp64", "achieved": m["tflops"], "peak": PEAK_FP64_VALU_TFLOPS,
-                     "unit": "TFLOP/s", "frac": m["tflops"] / PEAK_FP64_VALU_TFLOPS, "traffic": traffic,
+                   "relaxations_executed_fraction": m["executed_fraction"], "bit_exact": m["bit_exact"],
+                   "device": _lib.device_info()},
+        "roofline": {"bound": "valu_fp64", "achieved": m["tops_issued"], "peak": PEAK_FP64_VALU_TFLOPS,
+                     "unit": "TFLOP/s", "frac": fr["frac"], "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": m["kernel"], "launches_per_step": m["launches"],
-                     "avg_launch_ms": m["avg_launch_ms"], "flops_per_relaxation": 3,
+                     "avg_launch_ms": m["avg_launch_ms"],
+                     "ops_counted": "fp64 vector operations issued for the relaxations carried out",
                      "issued_ops_per_relaxation": m["issued_per_relaxation"],
-                     "frac_issued": m["tflops"] / 3.0 * m["issued_per_relaxation"] / PEAK_FP64_VALU_TFLOPS},
+                     "frac_reference_ops": fr["frac_reference_ops"], "reference_ops_per_relaxation": 3,
+                     "clock_ghz_under_load": m["clock_ghz"], "peak_clock_ghz": 2.4},
         "roofline_hbm": {"bound": "hbm", "achieved": m["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": m["gbs"] / PEAK_HBM_GBS, "traffic": traffic,
+                         "frac": fr["frac_hbm"], "traffic": traffic,
                          "algorithmic_bytes_per_launch": m["bytes_per_launch"]},
     }
     also = {}
     for w in [x for x in a.also.split(",") if x and x != a.workload]:
-        mm = measure(w, max(3, a.steps // 4), 1, host_leg=not a.headline_only)
+        mm = measure(w, max(3, a.steps // 4), 1, host_leg=not a.headline_only, check=True)
+        ff = fractions(mm)
         also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
                    "search_wall_ms_from_host_arrays": mm["host_ms"],
-                   "launch_scheme": mm["scheme"],
-                   "roofline_frac_valu_fp64": mm["tflops"] / PEAK_FP64_VALU_TFLOPS,
-                   "roofline_frac_hbm": mm["gbs"] / PEAK_HBM_GBS, "avg_launch_ms": mm["avg_launch_ms"]}
+                   "launch_scheme": mm["scheme"], "kernel": mm["kernel"], "register_tile": mm["tile"],
+                   "roofline_frac_valu_fp64": ff["frac"], "issued_ops_per_relaxation": mm["issued_per_relaxation"],
+                   "roofline_frac_valu_fp64_reference_ops": ff["frac_reference_ops"],
+                   "roofline_frac_hbm": ff["frac_hbm"], "avg_launch_ms": mm["avg_launch_ms"],
+                   "launches_per_step": mm["launches"], "bit_exact": mm["bit_exact"]}
     if also:
         line["also"] = also
     if a.row_skipping:
@@ -262,14 +390,18 @@ def main() -> int:
     if not a.headline_only:
         # The library's default additionally leaves out rows it can prove irrelevant (all-infinite sources /
         # unreachable from every start row); results are identical, fewer relaxations are carried out.
-        ms = measure(a.workload, max(3, a.steps // 2), 1, compute_all=False)
+        ms = measure(a.workload, max(3, a.steps // 2), 1, compute_all=False, check=True)
         line["with_row_skipping"] = {"value_nominal": ms["value"], "ms_per_step": ms["ms_per_step"],
                                      "relaxations_executed_fraction": ms["executed_fraction"],
-                                     "roofline_frac_valu_fp64_executed": ms["tflops"] / PEAK_FP64_VALU_TFLOPS}
-        mk = measure(a.workload, max(3, a.steps // 2), 1, keep_marks=True)
+                                     "roofline_frac_valu_fp64_executed": fractions(ms)["frac"],
+                                     "bit_exact": ms["bit_exact"]}
+        mk = measure(a.workload, max(3, a.steps // 2), 1, keep_marks=True, check=True)
         line["with_mark_table"] = {"value": mk["value"], "ms_per_step": mk["ms_per_step"],
-                                   "roofline_frac_valu_fp64": mk["tflops"] / PEAK_FP64_VALU_TFLOPS,
-                                   "algorithmic_bytes_per_launch": mk["bytes_per_launch"]}
+                                   "issued_ops_per_relaxation": mk["issued_per_relaxation"],
+                                   "roofline_frac_valu_fp64": fractions(mk)["frac"],
+                                   "roofline_frac_valu_fp64_reference_ops": fractions(mk)["frac_reference_ops"],
+                                   "algorithmic_bytes_per_launch": mk["bytes_per_launch"],
+                                   "bit_exact": mk["bit_exact"]}
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(a.workload)
         if "cfg3" in also:

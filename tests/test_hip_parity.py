@@ -23,10 +23,15 @@ def test_golden_small_full_arrays(golden, name):
     assert H.sha(mark) == rec["mark_sha256"], f"{name}: argmin table differs"
 
 
+def test_golden_covers_every_benchmark_config_on_the_gpu_box(golden):
+    """The same guard as the CPU suite's: every benchmark configuration has its vectors here too."""
+    for name in ["cfg0", "cfg1", "cfg2", "cfg4"] + [f"cfg3_{i:03d}" for i in range(256)]:
+        assert name in golden, name
+
+
 @pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4"])
 def test_golden_full_size(golden, name):
-    if name not in golden:
-        pytest.skip("fixture not generated")
+    assert name in golden, f"the committed vectors have no case {name}: a lost fixture is a failure, not a skip"
     rec = golden[name]
     inst = H.build_case(rec)
     H.assert_same_results(H.hip_solve(inst), H.golden_results(rec), name)
