@@ -1079,8 +1079,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // consecutive ones.  A window wider than the arithmetic of one layer reaches into the next
         // layer, whose workgroups can only wait, and they take the places of ones that could run on
         // CUs that then sit idle.  Dynamic LDS that the kernel never touches holds the number of
-        // workgroups per CU to (arithmetic-carrying block tasks of an average layer) / CUs, between 3
-        // and the 8 that fit anyway.
+        // workgroups per CU to just under (arithmetic-carrying block tasks of an average layer) / CUs,
+        // between 2 and the 8 that fit anyway.
         for (auto &seg : g.segments) {
             int64_t sum = 0, grid_rows = seg.layers;
             if (g.rows.empty()) {
@@ -1091,8 +1091,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 sum = sum * g.chunk / std::max<int64_t>(pairs, 1);
                 grid_rows = 1;
             }
-            int64_t per_cu = std::max<int64_t>(3, sum / grid_rows / std::max(pl->num_cu, 1));
-            if (pl->occupancy_cap_override >= 3) per_cu = pl->occupancy_cap_override;
+            // ... and strictly fewer than one layer's worth: with exactly a layer resident, all its workgroups
+            // start together, finish together, and the next layer's start together again, each paying the
+            // chain of dependent loads at its start with nothing to hide it behind; a narrower window
+            // makes layers overlap at their seams (measured, every cell computed, workgroups per CU ->
+            // ms: one instance L=32 S=44 V=65536, 4 per layer and CU: 3 -> 0.45, 4 -> 0.57, 5 -> 0.83, no
+            // limit 0.70; L=28 S=40 V=29493, 2.25 per layer and CU: 2 -> 0.38, 3 -> 0.55, no limit 0.53).
+            const int64_t cus = std::max(pl->num_cu, 1);
+            const int64_t per_layer = sum / grid_rows;
+            int64_t per_cu = std::max<int64_t>(2, (per_layer + cus - 1) / cus - 1);
+            if (pl->occupancy_cap_override >= 1) per_cu = pl->occupancy_cap_override;
             seg.lds_bytes = 0;
             if (per_cu < 8 && pl->lds_per_cu >= 65536 && !pl->no_occupancy_cap)
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);

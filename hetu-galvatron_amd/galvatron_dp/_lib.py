@@ -49,15 +49,21 @@ class UnsupportedInputError(ValueError):
     """Input outside what the device recurrence covers (a memory cost of 0)."""
 
 
+# The pointer members are declared as untyped pointers (same layout as the typed ones of the header):
+# they are then filled with plain addresses, which costs a fraction of a typed cast per array -- a sweep
+# builds thousands of these records.
+_ptr = ctypes.c_void_p
+
+
 class gdp_problem(ctypes.Structure):
     _fields_ = [("L", ctypes.c_int32), ("V", ctypes.c_int32), ("S", ctypes.c_int32),
-                ("mem", _i32p), ("intra", _f64p), ("inter", _f64p), ("inter_index", _i32p),
+                ("mem", _ptr), ("intra", _ptr), ("inter", _ptr), ("inter_index", _ptr),
                 ("n_inter", ctypes.c_int32), ("n_key", ctypes.c_int32),
-                ("other_mem", _i64p), ("other_time", _f64p), ("flags", ctypes.c_uint32)]
+                ("other_mem", _ptr), ("other_time", _ptr), ("flags", ctypes.c_uint32)]
 
 
 class gdp_result(ctypes.Structure):
-    _fields_ = [("total", _f64p), ("remaining", _i32p), ("res", _i32p), ("f_out", _f64p), ("mark_out", _i32p)]
+    _fields_ = [("total", _ptr), ("remaining", _ptr), ("res", _ptr), ("f_out", _ptr), ("mark_out", _ptr)]
 
 
 class gdp_timing(ctypes.Structure):
@@ -172,16 +178,12 @@ class Problem:
         self.res = np.full((self.n_key, self.L), -1, dtype=np.int32)
         self.f_out = np.empty((self.V, self.S), dtype=np.float64) if export_f else None
         self.mark_out = np.empty((self.L, self.V, self.S), dtype=np.int32) if export_mark else None
+        addr = lambda a: None if a is None else a.__array_interface__['data'][0]       # noqa: E731
         self._c_problem = gdp_problem(
-            self.L, self.V, self.S, self.mem.ctypes.data_as(_i32p), self.intra.ctypes.data_as(_f64p),
-            self.inter.ctypes.data_as(_f64p),
-            None if self.inter_index is None else self.inter_index.ctypes.data_as(_i32p),
-            int(self.inter.shape[0]), self.n_key, self.other_mem.ctypes.data_as(_i64p),
-            self.other_time.ctypes.data_as(_f64p), self.flags)
-        self._c_result = gdp_result(
-            self.total.ctypes.data_as(_f64p), self.remaining.ctypes.data_as(_i32p), self.res.ctypes.data_as(_i32p),
-            None if self.f_out is None else self.f_out.ctypes.data_as(_f64p),
-            None if self.mark_out is None else self.mark_out.ctypes.data_as(_i32p))
+            self.L, self.V, self.S, addr(self.mem), addr(self.intra), addr(self.inter), addr(self.inter_index),
+            int(self.inter.shape[0]), self.n_key, addr(self.other_mem), addr(self.other_time), self.flags)
+        self._c_result = gdp_result(addr(self.total), addr(self.remaining), addr(self.res), addr(self.f_out),
+                                    addr(self.mark_out))
 
     @property
     def relaxations(self) -> int:

@@ -23,6 +23,7 @@ import numpy as np
 
 __all__ = ["ModelArgs", "TrainArgs", "ParallelArgs", "ProfileModelArgs", "ProfileHardwareArgs",
            "MemoryCostModel", "TimeCostModel", "OtherTimeCostModel", "pipeline_costmodel",
+           "memory_cost_rows", "time_cost_rows", "NotVectorisable",
            "chunk_like_torch", "get_real_chunk", "get_time_cost_all_stages", "form_strategy",
            "strategy_str2list"]
 
@@ -205,6 +206,51 @@ def _zero_ratios(chunks, mixed_precision, async_grad_reduce):
 
 
 # ---- memory -----------------------------------------------------------------------------------------
+def _other_memory(strategy, chunks, zero2_ratio, zero3_ratio, global_batch_size, min_tp, max_tp, vsp, embed_sdp, train_args,
+                  parallel_args, profile):
+    """{vocab tp degree: [MB per pipeline stage]} of embedding / head / context
+    (cost_model.py:140-210)."""
+    pp, tp, dp = strategy[0], strategy[1], strategy[2]
+    off, on = profile.other_memory_pp_off, profile.other_memory_pp_on
+    if parallel_args.disable_vtp:
+        degrees = [1]
+    else:
+        degrees, k = [], min_tp
+        while k * pp <= strategy[0] * strategy[1] * strategy[2] and k <= max_tp:
+            degrees.append(k)
+            k *= 2
+    degrees = [k for k in degrees if k in off['model_states'].keys()
+               and k in on['first_stage']['model_states'] and k in on['last_stage']['model_states']]
+    out = {}
+    for k in degrees:
+        per_stage = [0] * pp
+        samples = global_batch_size * k / tp / dp
+        samples /= chunks
+        if vsp:
+            states_key, shard = 1, tp * dp
+        else:
+            states_key, shard = k, tp * dp // k
+        if embed_sdp:
+            ratio = zero3_ratio(shard)
+        else:
+            ratio = zero2_ratio(shard) if parallel_args.use_zero2_for_dp else 1.0
+        if pp == 1:
+            per_stage[0] += off['model_states'][states_key] * ratio + off['activation'][k] * samples
+        else:
+            if parallel_args.pipeline_type == 'pipedream_flush':
+                first, last = samples * pp, samples * 1
+            else:
+                first = last = samples
+            per_stage[0] += (on['first_stage']['model_states'][states_key] * ratio
+                             + on['first_stage']['activation'][k] * first)
+            per_stage[-1] += (on['last_stage']['model_states'][states_key] * ratio
+                              + on['last_stage']['activation'][k] * last)
+        for i in range(len(per_stage)):
+            per_stage[i] += train_args.pytorch_context_mem
+        out[k] = per_stage
+    return out
+
+
 class MemoryCostModel:
     """Memory (MB) of one layer under one strategy, and of the non-layer parts of the model per
     pipeline stage and vocabulary-tensor-parallel degree (cost_model.py:10-219)."""
@@ -271,52 +317,144 @@ class MemoryCostModel:
 
     def _other_memory(self, strategy, global_batch_size, min_tp, max_tp, vsp, embed_sdp, train_args, parallel_args,
                       profile):
-        """{vocab tp degree: [MB per pipeline stage]} of embedding / head / context
-        (cost_model.py:140-210)."""
-        pp, tp, dp = self.pp_size, self.tp_size, self.dp_size
-        off, on = profile.other_memory_pp_off, profile.other_memory_pp_on
-        if parallel_args.disable_vtp:
-            degrees = [1]
-        else:
-            degrees, k = [], min_tp
-            while k * pp <= strategy[0] * strategy[1] * strategy[2] and k <= max_tp:
-                degrees.append(k)
-                k *= 2
-        degrees = [k for k in degrees if k in off['model_states'].keys()
-                   and k in on['first_stage']['model_states'] and k in on['last_stage']['model_states']]
-        out = {}
-        for k in degrees:
-            per_stage = [0] * pp
-            samples = global_batch_size * k / tp / dp
-            samples /= self.chunks
-            if vsp:
-                states_key, shard = 1, tp * dp
-            else:
-                states_key, shard = k, tp * dp // k
-            if embed_sdp:
-                ratio = self.zero3_ratio(shard)
-            else:
-                ratio = self.zero2_ratio(shard) if parallel_args.use_zero2_for_dp else 1.0
-            if pp == 1:
-                per_stage[0] += off['model_states'][states_key] * ratio + off['activation'][k] * samples
-            else:
-                if parallel_args.pipeline_type == 'pipedream_flush':
-                    first, last = samples * pp, samples * 1
-                else:
-                    first = last = samples
-                per_stage[0] += (on['first_stage']['model_states'][states_key] * ratio
-                                 + on['first_stage']['activation'][k] * first)
-                per_stage[-1] += (on['last_stage']['model_states'][states_key] * ratio
-                                  + on['last_stage']['activation'][k] * last)
-            for i in range(len(per_stage)):
-                per_stage[i] += train_args.pytorch_context_mem
-            out[k] = per_stage
-        return out
+        return _other_memory(strategy, self.chunks, self.zero2_ratio, self.zero3_ratio, global_batch_size, min_tp,
+                             max_tp, vsp, embed_sdp, train_args, parallel_args, profile)
 
     def get_memory_cost(self):
         return {'parameter': self.parameter_size, 'model_states': self.model_states_size,
                 'activation': self.activation_size, 'enc_total': self.model_states_size + self.activation_size,
                 'other': self.other_memory_cost}
+
+
+# ---- memory of a whole strategy set at once ---------------------------------------------------------
+class NotVectorisable(Exception):
+    """The array forms below cover the inputs the search engine produces; anything else (a lane
+    without samples, a micro-batch split that does not give the asked count, a tensor-parallel degree
+    the profile has no entry for ...) is left to the per-strategy classes, which then compute or
+    raise exactly as the reference does."""
+
+
+_STRATEGY_ARRAYS = {}
+
+
+def _strategy_arrays(strategies):
+    """pp / tp / dp and the flags of a strategy list as arrays, kept per list (a sweep evaluates the
+    same few lists thousands of times)."""
+    key = tuple((int(s[0]), int(s[1]), int(s[2]), tuple(sorted(s[-1].items()))) for s in strategies)
+    hit = _STRATEGY_ARRAYS.get(key)
+    if hit is None:
+        flags = [s[-1] for s in strategies]
+        tp = np.array([s[1] for s in strategies], dtype=np.int64)
+        dp = np.array([s[2] for s in strategies], dtype=np.int64)
+        ulysses = np.array([f.get('sp', 0) == 1 for f in flags], dtype=bool)
+        hit = {"pp": np.array([s[0] for s in strategies], dtype=np.int64), "tp": tp, "dp": dp, "ulysses": ulysses,
+               "sdp": np.where(ulysses, tp * dp, dp),
+               "fsdp": np.array([bool(f.get('fsdp', 0)) for f in flags], dtype=bool),
+               "fsdp_off": np.array([('fsdp' in f and f['fsdp'] == 0) for f in flags], dtype=bool),
+               "cpt": np.array([bool(f.get('cpt', 0)) for f in flags], dtype=bool)}
+        if len(_STRATEGY_ARRAYS) > 4096:
+            _STRATEGY_ARRAYS.clear()
+        _STRATEGY_ARRAYS[key] = hit
+    return hit
+
+
+def _zero_ratio_arrays(chunks, d, mixed_precision, async_grad_reduce):
+    """(zero2, zero3) of ``_zero_ratios`` for arrays of micro-batch counts and sharding degrees, the
+    same expressions term by term."""
+    shard = 1 / d + 0.003
+    if mixed_precision:
+        one = (7 / 8 * shard + 1 / 8, shard)
+        many = (6 / 8 * shard + 2 / 8, 7 / 8 * shard + 1 / 8) if async_grad_reduce else \
+            ((7 / 8 * shard + 1 / 8) * 5 / 4, shard * 5 / 4)
+    else:
+        one = (3 / 4 * shard + 1 / 4, shard)
+        many = (2 / 4 * shard + 2 / 4, 3 / 4 * shard + 1 / 4) if async_grad_reduce else \
+            (3 / 4 * shard + 1 / 4, shard * 5 / 4)
+    single = chunks == 1
+    return np.where(single, one[0], many[0]), np.where(single, one[1], many[1])
+
+
+def memory_cost_rows(strategies, global_batch_size, mbsz, min_tp, max_tp, stage_idx=0, vsp=0, embed_sdp=False,
+                     model_args=None, train_args=None, parallel_args=None, profile_model_args=None):
+    """``MemoryCostModel(s, ...).get_memory_cost()`` for every strategy of a list in array
+    arithmetic: returns ``(enc_total float64 [S], other)`` with ``other`` the first strategy's
+    ``'other'`` entry (all that DpOnModel reads, dynamic_programming.py:254-288).  ``stage_idx`` may
+    be a sequence of pipeline stages: ``enc_total`` is then [stages, S] (``other`` is taken with the
+    first of them).  Each element is
+    produced by the same operations in the same order as the class (cost_model.py:10-219), hence the
+    same bits; raises ``NotVectorisable`` where the class would take a path this form does not cover."""
+    S = len(strategies)
+    if S == 0:
+        raise NotVectorisable
+    A = _strategy_arrays(strategies)
+    pp, tp, dp, ulysses, sdp = A["pp"], A["tp"], A["dp"], A["ulysses"], A["sdp"]
+    if mbsz <= -1 or min_tp <= 0 or (tp // min_tp < 1).any() or (tp * dp // min_tp < 1).any():
+        raise NotVectorisable
+
+    asked = parallel_args.chunks
+    if asked is None:
+        asked = np.array([parallel_args.optimal_chunk_func(global_batch_size // s[2], s, mbsz, min_tp)
+                          for s in strategies], dtype=np.float64)
+    else:
+        asked = np.full(S, asked, dtype=np.float64)
+    cap = global_batch_size // (tp * dp // min_tp)
+    cap = np.where(cap == 0, 1, cap)
+    chunks = np.where(asked > cap, cap, asked).astype(np.int64)           # int() of the class: towards zero
+    if (chunks < 1).any():
+        raise NotVectorisable
+
+    # the split torch.arange(size).chunk(chunks) gives: pieces of `step` until the range is used up
+    size = (global_batch_size / dp / (tp // min_tp)).astype(np.int64)
+    if (size < 1).any():
+        raise NotVectorisable
+    step = (size + chunks - 1) // chunks
+    pieces = (size + step - 1) // step
+    first_piece = np.minimum(step, size)
+    bsz = global_batch_size / dp
+    one_f_one_b = (pp == 1) | (parallel_args.pipeline_type == 'pipedream_flush')
+    if one_f_one_b.any():
+        if (pieces != chunks)[one_f_one_b].any():
+            raise NotVectorisable                                          # the class asserts here
+        stage = np.asarray(stage_idx, dtype=np.int64)
+        left = pp - (stage[:, None] if stage.ndim == 1 else stage)
+        in_flight = np.where(left <= chunks, left, chunks)
+        if (in_flight < 1)[..., one_f_one_b].any():
+            raise NotVectorisable
+        ratio = np.minimum(in_flight * step, size) / size                   # sum of the first pieces / sum of all
+        bsz = np.where(one_f_one_b, ratio * bsz, first_piece)
+    else:
+        bsz = first_piece.astype(np.float64)
+        if np.ndim(stage_idx) == 1:
+            bsz = np.broadcast_to(bsz, (len(stage_idx), S))
+
+    zero2, zero3 = _zero_ratio_arrays(chunks, sdp, train_args.mixed_precision, train_args.async_grad_reduce)
+    parameter = np.where(ulysses, model_args.parameter_size, model_args.parameter_size / tp)
+    states = 4 * parameter
+    if parallel_args.use_zero2_for_dp:
+        states = np.where(A["fsdp"], states * zero3, np.where(A["fsdp_off"], states * zero2, states))
+    else:
+        states = np.where(A["fsdp"], states * zero3, states)
+
+    per_sample = profile_model_args.tp_activation_per_bsz_dict
+    cpt = A["cpt"]
+    if cpt.any() and per_sample.get('checkpoint') is None:
+        raise NotVectorisable
+    if any(int(t) not in per_sample for t in tp[~cpt]):
+        raise NotVectorisable
+    plain = np.array([per_sample[int(t)] if not c else 0.0 for t, c in zip(tp, cpt)], dtype=np.float64) * bsz
+    if cpt.any():
+        kept = per_sample['checkpoint'] * bsz
+        if parallel_args.sequence_parallel:
+            kept = kept / tp
+        activation = np.where(cpt, kept, plain)
+    else:
+        activation = plain
+
+    s0 = strategies[0]
+    z2, z3 = _zero_ratios(int(chunks[0]), train_args.mixed_precision, train_args.async_grad_reduce)
+    other = _other_memory(s0, int(chunks[0]), z2, z3, global_batch_size, min_tp, max_tp, vsp, embed_sdp, train_args,
+                          parallel_args, profile_model_args)
+    return states + activation, other
 
 
 # ---- time -------------------------------------------------------------------------------------------
@@ -456,6 +594,118 @@ class TimeCostModel:
         return result / self.layer_num
 
 
+def time_cost_rows(strategies, global_batch_size, no_comm=False, model_args=None, train_args=None, parallel_args=None,
+                   profile_model_args=None, profile_hardware_args=None):
+    """``TimeCostModel(s, global_batch_size, ...).gen_result()`` for every strategy of a list in
+    array arithmetic (float64 [S]); the same operations in the same order as the class
+    (cost_model.py:221-466), table look-ups per strategy, everything else elementwise.  Raises
+    ``NotVectorisable`` where the class would raise or take a path not covered here."""
+    S = len(strategies)
+    if S == 0:
+        raise NotVectorisable
+    if model_args.layer_num is None:
+        model_args.layer_num = 24                       # as the class: written back into the caller's record
+    hw = profile_hardware_args
+    mixed = train_args.mixed_precision
+    layer_num, seq_len, hidden = model_args.layer_num, model_args.seq_length, model_args.hidden_size
+    A = _strategy_arrays(strategies)
+    pp, tp, dp, ulysses, sdp, fsdp, cpt = A["pp"], A["tp"], A["dp"], A["ulysses"], A["sdp"], A["fsdp"], A["cpt"]
+    bsz = global_batch_size / dp
+    parameter = np.where(ulysses, model_args.parameter_size, model_args.parameter_size / tp)
+
+    per_layer = profile_model_args.forward_computation_time
+    if isinstance(per_layer, np.ndarray):
+        fct = _line(bsz / tp, per_layer) * layer_num
+    else:
+        fct = per_layer * bsz / tp * layer_num
+    bct = fct * hw.bct_fct_coe
+    bct = np.where(cpt, bct + fct, bct)
+
+    dp_message = (2 * (dp - 1) / dp * parameter) * layer_num
+    if mixed:
+        dp_message = dp_message / 2
+    allgather = dp_message * 0.5
+    if no_comm:
+        dp_message = np.zeros(S)
+
+    # per-strategy look-ups: coefficients of the gradient and activation collectives
+    dc, tc, per_message = np.empty(S), np.zeros(S), np.zeros(S)
+    tp_sp = parallel_args.sp_space == 'tp+sp'
+    word = 2 if mixed else 4
+    try:
+        for i, st in enumerate(strategies):
+            t, d = int(tp[i]), int(dp[i])
+            both = not (t == 1 or d == 1)
+            if both and not ulysses[i] or (both and not tp_sp):
+                consecutive = st[-1]['tp']
+                if consecutive not in (0, 1):
+                    raise NotVectorisable
+            if ulysses[i]:
+                dc[i] = _group_coe(hw.comm_coe_dict, int(sdp[i]))
+            elif not both:
+                dc[i] = _group_coe(hw.comm_coe_dict, d)
+            else:
+                dc[i] = _group_coe(hw.comm_coe_dict, d, 0 if consecutive else 1)
+            if tp_sp:
+                if t > 1:
+                    table = (hw.all2all_dict if ulysses[i] else hw.allreduce_dict)[t]
+                    size = bsz[i] * seq_len * hidden * word
+                    per_message[i] = table[size] if size in table else _line(1 / 1024 / 1024 * size, table["popt"])
+            elif not both:
+                tc[i] = _group_coe(hw.comm_coe_dict, t)
+            else:
+                tc[i] = _group_coe(hw.comm_coe_dict, t, 1 if consecutive else 0)
+    except (KeyError, TypeError):
+        raise NotVectorisable from None
+    dc_overlap = dc * hw.dp_overlap_coe
+
+    if tp_sp:
+        comm_num = np.where(cpt, 4 * layer_num * 1.5, 4 * layer_num)
+        tp_time = comm_num * per_message
+    else:
+        volume = 2 * (tp - 1) / tp * (bsz * seq_len * hidden * 4 * 4 / 1024 / 1024) * layer_num
+        volume = np.where(cpt, volume * 1.5, volume)
+        if mixed:
+            volume = volume / 2
+        tp_time = volume * tc
+
+    def overlap(message, backward):
+        """bct_dp_overlap of the class, both of its return values."""
+        comm = message * dc_overlap
+        comp = backward * hw.bct_overlap_coe
+        with np.errstate(divide='ignore', invalid='ignore'):
+            more_comm = (message - comp / dc_overlap) * dc
+            more_comp = backward - comm / hw.bct_overlap_coe
+        first = np.where(comm > comp, comp, np.where(comm < comp, comm, comp))
+        rest = np.where(comm > comp, more_comm, np.where(comm < comp, more_comp, 0.0))
+        return first, rest
+
+    o_full, r_full = overlap(dp_message, bct)
+    o_half, r_half = overlap(dp_message, bct * 1 / 2)
+    extra = hw.extra_overhead
+    only_dp = (tp == 1) & (dp > 1)
+    only_tp = (dp == 1) & (tp > 1)
+    neither = (dp == 1) & (tp == 1)
+    narrow_tp = tp < tp * dp // 2
+    result = np.where(only_dp, fct + o_full + r_full + extra,
+             np.where(only_tp, fct + bct + tp_time,
+             np.where(neither, fct + bct,
+             np.where(narrow_tp, fct + o_full + r_full + tp_time + extra,
+                      fct + 1 / 2 * bct + o_half + r_half + tp_time + extra))))
+    result = np.where(fsdp, result + allgather * dc * 1, result)
+    if hw.p2p_comm_coe_dict is not None and (pp > 1).any():
+        try:
+            coe = np.array([hw.p2p_comm_coe_dict[int(x)] if x > 1 else 0.0 for x in pp])
+        except KeyError:
+            raise NotVectorisable from None
+        message = pp * 2 * bsz * seq_len * hidden * 4 / 1024 / 1024
+        if mixed:
+            message = message / 2
+        result = np.where(pp > 1, result + message * coe, result)
+    result = result * (0.001 * hw.costmodel_coe)
+    return result / layer_num
+
+
 class OtherTimeCostModel:
     """Time (s) of the non-layer parts of the model (embedding, head) per pipeline stage and vocabulary
     tensor-parallel degree, with and without the gradient all-reduce (cost_model.py:468-658)."""
@@ -588,18 +838,30 @@ def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_arg
         max_chunk = chunks
     pp_deg = len(partition)
 
-    texts = list(set(form_strategy(s) for s in strategies))
+    names = [form_strategy(s) for s in strategies]
+    texts = list(set(names))
     full, compute_only = {}, {}
     for t in range(len(layer_num_list)):
         common = dict(model_args=model_args_list[t], train_args=train_args_list[t], parallel_args=parallel_args_list[t],
                       profile_model_args=profile_model_args_list[t],
-                      profile_hardware_args=profile_hardware_args_list[t], logger=logger)
-        for text in texts:
-            full[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], **common).gen_result()
-            compute_only[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], no_comm=True,
+                      profile_hardware_args=profile_hardware_args_list[t])
+        rows = None
+        if timecostmodel is TimeCostModel:              # this package's own model: all strategies at once
+            try:
+                parsed = [strategy_str2list(text) for text in texts]
+                rows = (time_cost_rows(parsed, bsz_per_chunk[t], **common),
+                        time_cost_rows(parsed, bsz_per_chunk[t], no_comm=True, **common))
+            except NotVectorisable:
+                rows = None
+        for n, text in enumerate(texts):
+            if rows is not None:
+                full[t, text], compute_only[t, text] = rows[0][n], rows[1][n]
+                continue
+            full[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], logger=logger, **common).gen_result()
+            compute_only[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], no_comm=True, logger=logger,
                                                   **common).gen_result()
-    per_layer_full = [full[type_of_layer[i], form_strategy(s)] for i, s in enumerate(strategies)]
-    per_layer_compute = [compute_only[type_of_layer[i], form_strategy(s)] for i, s in enumerate(strategies)]
+    per_layer_full = [full[type_of_layer[i], name] for i, name in enumerate(names)]
+    per_layer_compute = [compute_only[type_of_layer[i], name] for i, name in enumerate(names)]
     stage_full = get_time_cost_all_stages(per_layer_full, partition)
     stage_compute = get_time_cost_all_stages(per_layer_compute, partition)
     assert len(other_time_cost) == len(stage_compute)

@@ -56,6 +56,19 @@ class DPAlg:
         self.inter_cost = inter_layer_cost
         self.intra_cost = intra_layer_cost
 
+    def set_v_and_cost_shared(self, v: np.ndarray, intra_layer_cost: np.ndarray, inter_tables: np.ndarray,
+                              inter_index: np.ndarray):
+        """``set_v_and_cost`` for layers that share a few transition matrices: ``inter_tables`` [T,S,S]
+        and ``inter_index`` [L] instead of the dense [L,S,S] array (which would repeat each matrix once
+        per layer on the host, in the upload and in device memory).  Fine-grained mode only."""
+        assert self.fine_grained_mode
+        assert v.shape == (self.layer_num, self.strategy_num) and intra_layer_cost.shape == v.shape
+        assert inter_tables.ndim == 3 and inter_tables.shape[1:] == (self.strategy_num, self.strategy_num)
+        assert inter_index.shape == (self.layer_num,)
+        self.v_data = v.astype(np.int32)
+        self.inter_cost = galvatron_dp_core.SharedInter(inter_tables, inter_index)
+        self.intra_cost = intra_layer_cost
+
     # -- coarse mode: one strategy for the whole stage, closed form (dynamic_programming.py:62-75) ----
     def _fit_coarse(self):
         keys = list(self.other_mem_cost)
@@ -127,6 +140,81 @@ def _same_strategy(a, b, ignore=()):
     return True
 
 
+_INTER_STRUCTURES = {}
+
+
+def _inter_structure(strategy_set, sequence_parallel):
+    """What the pairwise inter-layer cost of a strategy set owes to the strategies alone
+    (dynamic_programming.py:292-367): ``big`` max(tp_i, tp_j); ``redistribute`` the pairs whose
+    activations have to be re-laid out; ``coe_picks`` [(group size, layout flag or None, mask)] naming the
+    collective coefficient each pair takes; ``bias`` / ``has_bias`` the tiny ordering biases between
+    strategies that differ only in sp / fsdp / cpt, later rules overriding earlier ones as in the
+    reference.  Kept per strategy set (a sweep builds the same few sets hundreds of times)."""
+    key = (tuple((int(st[0]), int(st[1]), int(st[2]), tuple(sorted(st[-1].items()))) for st in strategy_set),
+           sequence_parallel)
+    hit = _INTER_STRUCTURES.get(key)
+    if hit is not None:
+        return hit
+    S = len(strategy_set)
+    tp = np.array([s[1] for s in strategy_set], dtype=np.int64)
+    dp = np.array([s[2] for s in strategy_set], dtype=np.int64)
+    has_tp = np.array(['tp' in s[-1] for s in strategy_set])
+    tp_flag = np.array([s[-1].get('tp', -1) for s in strategy_set], dtype=np.int64)
+    tp_i, tp_j = tp[:, None], tp[None, :]
+    both = has_tp[:, None] & has_tp[None, :]
+    differ = tp_flag[:, None] != tp_flag[None, :]
+    redistribute = tp_j > tp_i
+    redistribute |= both & (tp_j == tp_i) & differ
+    redistribute |= both & ((tp * dp)[:, None] == 8) & (tp_i == 4) & (tp_j == 2) & differ
+    if sequence_parallel:
+        redistribute |= tp_j != tp_i
+    big = np.maximum(tp_i, tp_j)
+    # communication coefficient of the wider of the two tensor-parallel groups: the plain one when
+    # that group is everything (or there is no data parallelism beside it), else by the layout
+    # flag of the strategy that owns the wider group
+    small_dp = np.minimum(dp[:, None], dp[None, :])
+    plain = (big == 1) | (small_dp == 1)
+    owner_flag = np.where(tp_j > tp_i, tp_flag[None, :], tp_flag[:, None])
+    assert np.isin(owner_flag[~plain], (0, 1)).all()
+    coe_picks = []
+    for t in np.unique(big):
+        t = int(t)
+        here = big == t
+        if (here & plain).any():
+            coe_picks.append((t, None, here & plain))
+        for flag in (0, 1):
+            pick = here & ~plain & (owner_flag == flag)
+            if pick.any():
+                coe_picks.append((t, flag, pick))
+
+    # "Same apart from key k" (the reference's match_strategy, dynamic_programming.py:196-210) is
+    # equality of (pp, tp, dp) and of the option dictionaries with k removed.
+    def same_apart_from(*ignore):
+        ids, seen = [], {}
+        for st in strategy_set:
+            k = (tuple(int(x) for x in st[:3]), frozenset((a, b) for a, b in st[-1].items() if a not in ignore))
+            ids.append(seen.setdefault(k, len(seen)))
+        ids = np.array(ids)
+        return ids[:, None] == ids[None, :]
+
+    on = lambda name: np.array([bool(st[-1].get(name)) for st in strategy_set])       # noqa: E731
+    sp_j, fsdp_j, cpt_j, fsdp_i = on('sp')[None, :], on('fsdp')[None, :], on('cpt')[None, :], on('fsdp')[:, None]
+    off_diagonal = ~np.eye(S, dtype=bool)
+    only_fsdp, only_cpt, both_keys = same_apart_from('fsdp'), same_apart_from('cpt'), same_apart_from('fsdp', 'cpt')
+    bias = np.full((S, S), np.nan)
+    bias[off_diagonal & same_apart_from('sp') & sp_j] = 1e-10
+    bias[off_diagonal & only_fsdp & fsdp_j] = 1e-9
+    bias[off_diagonal & only_cpt & cpt_j] = 2e-9
+    bias[off_diagonal & both_keys & fsdp_j & cpt_j] = 3e-9
+    bias[off_diagonal & both_keys & ~only_fsdp & ~only_cpt & fsdp_i & cpt_j] = 1e-9
+    hit = {"big": big, "redistribute": redistribute, "coe_picks": coe_picks, "has_bias": ~np.isnan(bias),
+           "bias": np.nan_to_num(bias)}
+    if len(_INTER_STRUCTURES) > 4096:
+        _INTER_STRUCTURES.clear()
+    _INTER_STRUCTURES[key] = hit
+    return hit
+
+
 class _Prepared:
     """Everything one pipeline degree contributes to the batch: the DP instances of its stages and
     what is needed to turn their results into the reference's return tuple."""
@@ -194,106 +282,106 @@ class DpOnModel:
                     parallel_args=self.parallel_args_list[i], profile_model_args=self.profile_model_args_list[i])
 
     def _intra_cost(self, strategy_set, bsz, chunks):
-        """[L,S] time of a layer under each strategy (dynamic_programming.py:228-245)."""
+        """[L,S] time of a layer under each strategy (dynamic_programming.py:228-245).  With this
+        package's own time model the S values of a layer type come out of one array evaluation
+        (``cost_models.time_cost_rows``, the same bits); any other model is called per strategy."""
         blocks = []
         for i, n in enumerate(self.layer_num):
             b = bsz / chunks[i] if self.model_microbatch_after_dp else bsz
-            row = [self.timecost_model(s, b, profile_hardware_args=self.profile_hardware_args_list[i],
-                                       logger=self.logger, **self._model_kwargs(i)).gen_result() for s in strategy_set]
+            row = None
+            if self.timecost_model is cost_models.TimeCostModel:
+                try:
+                    row = cost_models.time_cost_rows(strategy_set, b,
+                                                     profile_hardware_args=self.profile_hardware_args_list[i],
+                                                     **self._model_kwargs(i))
+                except cost_models.NotVectorisable:
+                    row = None
+            if row is None:
+                row = [self.timecost_model(s, b, profile_hardware_args=self.profile_hardware_args_list[i],
+                                           logger=self.logger, **self._model_kwargs(i)).gen_result() for s in strategy_set]
             blocks.append(np.array(row, dtype=np.float64).reshape(1, -1).repeat(n, axis=0))
         return np.concatenate(blocks, axis=0)
+
+    def _memory_rows(self, strategy_set, i, bsz, mbsz, min_tp, max_tp, vsp, embed_sdp, stage_ids):
+        """(enc_total [stages, S], 'other' of the first strategy on the first stage) for layer type
+        ``i``: one array evaluation with this package's own memory model, one object per strategy and
+        stage otherwise.  ``stage_ids`` is ``[None]`` where the stage does not matter (gpipe)."""
+        if self.memcost_model is cost_models.MemoryCostModel:
+            try:
+                rows, other = cost_models.memory_cost_rows(
+                    strategy_set, bsz, mbsz, min_tp, max_tp, vsp=vsp, embed_sdp=embed_sdp,
+                    stage_idx=[0 if x is None else x for x in stage_ids], **self._model_kwargs(i))
+                return rows, other
+            except cost_models.NotVectorisable:
+                pass
+        rows, other = [], None
+        for stage_idx in stage_ids:
+            extra = {} if stage_idx is None else {"stage_idx": stage_idx}
+            costs = [self.memcost_model(s, bsz, mbsz=mbsz, min_tp=min_tp, max_tp=max_tp, vsp=vsp, embed_sdp=embed_sdp,
+                                        logger=self.logger, **extra, **self._model_kwargs(i)).get_memory_cost()
+                     for s in strategy_set]
+            rows.append([c['enc_total'] for c in costs])
+            if other is None:
+                other = costs[0]['other']
+        return np.array(rows), other
 
     def _memory_cost(self, strategy_set, pp_deg, bsz, mbsz, min_tp, max_tp, vsp, embed_sdp):
         """Per-stage [L,S] memory tables (ceil MB, int32) and the ``other`` memory of the first layer
         type (dynamic_programming.py:254-288)."""
         other_mem_cost = {}
         stage_ids = [None] if self.pipeline_type == "gpipe" else list(range(pp_deg))
-        tables = []
-        for stage_idx in stage_ids:
-            blocks = []
-            for i, n in enumerate(self.layer_num):
-                extra = {} if stage_idx is None else {"stage_idx": stage_idx}
-                costs = [self.memcost_model(s, bsz, mbsz=mbsz, min_tp=min_tp, max_tp=max_tp, vsp=vsp,
-                                            embed_sdp=embed_sdp, logger=self.logger, **extra,
-                                            **self._model_kwargs(i)).get_memory_cost() for s in strategy_set]
-                if i == 0 and stage_idx in (None, 0):
-                    for k, val in costs[0]['other'].items():
-                        other_mem_cost[k] = np.ceil(val).astype(int)
-                row = np.ceil(np.array([c['enc_total'] for c in costs])).astype(np.int32)
-                blocks.append(row.reshape(1, -1).repeat(n, axis=0))
-            tables.append(np.concatenate(blocks, axis=0))
+        per_type = []
+        for i, n in enumerate(self.layer_num):
+            enc_total, other = self._memory_rows(strategy_set, i, bsz, mbsz, min_tp, max_tp, vsp, embed_sdp, stage_ids)
+            if i == 0:
+                for k, val in other.items():
+                    other_mem_cost[k] = np.ceil(val).astype(int)
+            per_type.append(np.ceil(enc_total).astype(np.int32))          # [stages, S]
+        tables = [np.concatenate([rows[j].reshape(1, -1).repeat(n, axis=0) for rows, n in zip(per_type, self.layer_num)],
+                                 axis=0) for j in range(len(stage_ids))]
         if self.pipeline_type == "gpipe":
             return [tables[0]] * pp_deg, other_mem_cost
         return tables, other_mem_cost
 
     def _inter_matrix(self, strategy_set, idx, mbsz, min_tp):
         """[S,S] cost of switching from strategy i (row) to strategy j (column) between two layers
-        of type ``idx`` (dynamic_programming.py:292-367), built from per-strategy feature vectors."""
-        S = len(strategy_set)
-        tp = np.array([s[1] for s in strategy_set], dtype=np.int64)
-        dp = np.array([s[2] for s in strategy_set], dtype=np.int64)
-        has_tp = np.array(['tp' in s[-1] for s in strategy_set])
-        tp_flag = np.array([s[-1].get('tp', -1) for s in strategy_set], dtype=np.int64)
-        tp_i, tp_j = tp[:, None], tp[None, :]
-        both = has_tp[:, None] & has_tp[None, :]
-        differ = tp_flag[:, None] != tp_flag[None, :]
-        redistribute = tp_j > tp_i
-        redistribute |= both & (tp_j == tp_i) & differ
-        redistribute |= both & ((tp * dp)[:, None] == 8) & (tp_i == 4) & (tp_j == 2) & differ
-        if self.config.sequence_parallel:
-            redistribute |= tp_j != tp_i
+        of type ``idx`` (dynamic_programming.py:292-367).  What depends on the strategies alone --
+        which pairs redistribute, which collective coefficient a pair takes, which pairs get one of
+        the tiny ordering biases -- is worked out once per strategy set (``_inter_structure``, kept
+        for the whole sweep); a call adds the volumes and coefficients."""
+        st = _inter_structure(strategy_set, bool(self.config.sequence_parallel))
+        big = st["big"]
         sample_num = self.sequence_len[idx] * self.config.hidden_size * (4 if self.config.mixed_precision == "fp32" else 2)
-        big = np.maximum(tp_i, tp_j)
         volume = (big - 1) / big * mbsz * (big // min_tp) * sample_num      # same order of operations
-        cost = np.where(redistribute, volume, 0.0)
-        # communication coefficient of the wider of the two tensor-parallel groups: the plain one when
-        # that group is everything (or there is no data parallelism beside it), else by the layout
-        # flag of the strategy that owns the wider group
-        small_dp = np.minimum(dp[:, None], dp[None, :])
-        plain = (big == 1) | (small_dp == 1)
-        owner_flag = np.where(tp_j > tp_i, tp_flag[None, :], tp_flag[:, None])
-        assert np.isin(owner_flag[~plain], (0, 1)).all()
-        coe = np.empty((S, S), dtype=np.float64)
+        cost = np.where(st["redistribute"], volume, 0.0)
+        coe = np.empty(big.shape, dtype=np.float64)
         table = self.comm_coe_dict
-        for t in np.unique(big):
-            t = int(t)
-            here = big == t
-            if (here & plain).any():
-                coe[here & plain] = table['%d' % t] if '%d' % t in table else table['%d_1' % t]
-            for flag in (0, 1):
-                pick = here & ~plain & (owner_flag == flag)
-                if pick.any():
-                    coe[pick] = table['%d_%d' % (t, flag)]
+        for t, flag, pick in st["coe_picks"]:
+            if flag is None:
+                coe[pick] = table['%d' % t] if '%d' % t in table else table['%d_1' % t]
+            else:
+                coe[pick] = table['%d_%d' % (t, flag)]
         cost = cost * coe * 1e-7
-        # tiny ordering biases between strategies that differ only in sp / fsdp / cpt.  "Same apart
-        # from key k" (the reference's match_strategy, dynamic_programming.py:196-210) is equality of
-        # (pp, tp, dp) and of the option dictionaries with k removed; the rules are applied in the
-        # reference's order, later ones overriding earlier ones.
-        def same_apart_from(*ignore):
-            ids, seen = [], {}
-            for st in strategy_set:
-                key = (tuple(int(x) for x in st[:3]), frozenset((k, v) for k, v in st[-1].items() if k not in ignore))
-                ids.append(seen.setdefault(key, len(seen)))
-            ids = np.array(ids)
-            return ids[:, None] == ids[None, :]
+        return np.where(st["has_bias"], st["bias"], cost)
 
-        on = lambda name: np.array([bool(st[-1].get(name)) for st in strategy_set])       # noqa: E731
-        sp_j, fsdp_j, cpt_j, fsdp_i = on('sp')[None, :], on('fsdp')[None, :], on('cpt')[None, :], on('fsdp')[:, None]
-        off_diagonal = ~np.eye(S, dtype=bool)
-        only_fsdp, only_cpt, both_keys = same_apart_from('fsdp'), same_apart_from('cpt'), same_apart_from('fsdp', 'cpt')
-        cost[off_diagonal & same_apart_from('sp') & sp_j] = 1e-10
-        cost[off_diagonal & only_fsdp & fsdp_j] = 1e-9
-        cost[off_diagonal & only_cpt & cpt_j] = 2e-9
-        cost[off_diagonal & both_keys & fsdp_j & cpt_j] = 3e-9
-        cost[off_diagonal & both_keys & ~only_fsdp & ~only_cpt & fsdp_i & cpt_j] = 1e-9
-        return cost
+    def _inter_tables(self, strategy_set, mbsz, min_tp):
+        """The transition matrices of one pipeline degree as the device takes them: ``tables``
+        [1 + layer types, S, S] -- matrix 0 is all zeros, for the first layer of the model, which has no
+        switch before it (dynamic_programming.py:372) -- and ``index`` [L] naming every layer's matrix."""
+        S = len(strategy_set)
+        tables = np.zeros((1 + len(self.layer_num), S, S), dtype=np.float64)
+        index = []
+        for idx, n in enumerate(self.layer_num):
+            tables[1 + idx] = self._inter_matrix(strategy_set, idx, mbsz, min_tp)
+            index += [1 + idx] * n
+        index = np.array(index, dtype=np.int32)
+        index[0] = 0
+        return tables, index
 
     def _inter_cost(self, strategy_set, mbsz, min_tp):
-        blocks = [np.expand_dims(self._inter_matrix(strategy_set, idx, mbsz, min_tp), 0).repeat(n, axis=0)
-                  for idx, n in enumerate(self.layer_num)]
-        inter = np.concatenate(blocks, axis=0)
-        inter[0, :, :] = 0                               # no switch before the first layer (:372)
-        return inter
+        """The same as one dense [L,S,S] array, the reference's layout (dynamic_programming.py:289-372)."""
+        tables, index = self._inter_tables(strategy_set, mbsz, min_tp)
+        return tables[index]
 
     def _global_memory(self, mbsz, min_tp, max_tp, sp_search, coarse):
         cfg = self.config
@@ -324,12 +412,13 @@ class DpOnModel:
             parallel_args=self.parallel_args_list[0], profile_model_args=self.profile_model_args_list[0],
             profile_hardware_args=self.profile_hardware_args_list[0], logger=self.logger).gen_result()
         v_stage, P.other_mem_cost = self._memory_cost(strategy_set, pp_deg, bsz, mbsz, min_tp, max_tp, vsp, embed_sdp)
-        inter = self._inter_cost(strategy_set, mbsz, min_tp)
+        tables, index = self._inter_tables(strategy_set, mbsz, min_tp)
         P.pp_stage_list = self.pp_stage_dict[pp_deg]
         P.coarse = self.config.fine_grained_mode == 0
         gmem = int(self._global_memory(mbsz, min_tp, max_tp, sp_search, P.coarse))
         P.dps, P.local_sets = [], []
         columns = [[si] for si in range(S)] if P.coarse else [list(range(S))]
+        inter = tables[index] if P.coarse else None      # dense only where single columns are cut out of it
         for cols in columns:                             # coarse mode: one single-strategy DP per strategy
             start = 0
             local = [strategy_set[c] for c in cols]
@@ -339,8 +428,11 @@ class DpOnModel:
                 other_time = {k: v[i] for k, v in P.other_time_cost[0].items()}
                 dp = DPAlg(self.max_mem, other_mem, other_time, n, len(cols), local, self.config.fine_grained_mode)
                 rows = slice(start, start + n)
-                dp.set_v_and_cost(v_stage[i][rows][:, cols], intra[rows][:, cols],
-                                  inter[rows][:, cols][:, :, cols])
+                if P.coarse:
+                    dp.set_v_and_cost(v_stage[i][rows][:, cols], intra[rows][:, cols],
+                                      inter[rows][:, cols][:, :, cols])
+                else:                                    # every stage of the pipeline degree shares the tables
+                    dp.set_v_and_cost_shared(v_stage[i][rows], intra[rows], tables, index[rows])
                 P.dps.append(dp)
                 start += n
             P.local_sets.append(local)

@@ -23,7 +23,7 @@ import os
 
 import numpy as np
 
-from . import cost_models, profile_configs
+from . import _lib, cost_models, profile_configs
 from .dynamic_programming import DPAlg, DpOnModel
 from .pp_utils import check_optimal_chunks, get_pp_stage_for_bsz, optimal_chunk_func_default
 
@@ -76,6 +76,7 @@ class SearchEngine:
         self.results = None
         self.optimal = None
         self.solved_instances = 0
+        self.keep_device_cache = False      # True: a sweep leaves the library's cached device allocations in place
 
     # ---- model, paths (search_engine.py:45-97) ---------------------------------------------------------
     def set_model(self, model_name, model_layer_configs, path=None):
@@ -413,6 +414,10 @@ class SearchEngine:
             for _, _, _, _, first, count, _ in pending:
                 fits += DPAlg.fit_many(all_dps[first:first + count])
         self.strategies = strategies_backup
+        if not self.keep_device_cache:
+            # the library keeps the device allocations of finished batches for the next one; a search is
+            # usually the last thing its process asks of the device, so they are handed back here
+            _lib.cache_trim()
 
         results = {}
         for bsz, chunk, min_tp, max_tp, vsp, embed_sdp in self.tasks():        # the reference's empty levels

@@ -19,7 +19,7 @@ import numpy as np
 
 from galvatron_dp import _lib
 
-__all__ = ["dynamic_programming_core", "dynamic_programming_core_batch", "set_export"]
+__all__ = ["dynamic_programming_core", "dynamic_programming_core_batch", "set_export", "SharedInter"]
 
 _export = False
 
@@ -31,15 +31,36 @@ def set_export(flag: bool) -> None:
     _export = bool(flag)
 
 
+class SharedInter:
+    """``inter_cost`` of a call whose layers share a few transition matrices: ``tables`` f64 [T,S,S]
+    and ``index`` int32 [L] (layer -> matrix), accepted wherever the plugin takes the reference's dense
+    [L,S,S] array (no counterpart in the reference, which always passes the dense array).  The device
+    then holds every matrix once."""
+    __slots__ = ("tables", "index")
+
+    def __init__(self, tables, index):
+        self.tables = np.ascontiguousarray(tables, dtype=np.float64)
+        self.index = np.ascontiguousarray(index, dtype=np.int32)
+
+    def dense(self):
+        return self.tables[self.index]
+
+    def __getitem__(self, item):               # so that code written for the dense array can still slice it
+        return self.dense()[item]
+
+
 def _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, other_mem_cost, other_time_cost,
              export):
     L, V, S = int(layer_num), int(max_mem), int(strategy_num)
     mem = np.ascontiguousarray(v_data, dtype=np.int32).reshape(L, S)
     intra = np.ascontiguousarray(intra_cost, dtype=np.float64).reshape(L, S)
-    inter = np.ascontiguousarray(inter_cost, dtype=np.float64).reshape(L, S, S)
     keys = sorted(int(k) for k in other_mem_cost)          # std::map iterates in ascending key order
     om = [int(other_mem_cost[k]) for k in keys]
     ot = [float(other_time_cost[k]) if k in other_time_cost else 0.0 for k in keys]  # map::operator[] default
+    if isinstance(inter_cost, SharedInter):
+        return keys, _lib.Problem(mem, intra, inter_cost.tables.reshape(-1, S, S), V, om, ot,
+                                  inter_index=inter_cost.index.reshape(L), export_f=export, export_mark=export)
+    inter = np.ascontiguousarray(inter_cost, dtype=np.float64).reshape(L, S, S)
     return keys, _lib.Problem(mem, intra, inter, V, om, ot, export_f=export, export_mark=export)
 
 

@@ -162,3 +162,78 @@ def test_pipeline_model_degenerate_cases():
     one = M.TimeCostModel(s, 64, **a).gen_result()
     compute = M.TimeCostModel(s, 64, no_comm=True, **a).gen_result()
     assert total == np.sum([compute] * 3) + max(np.sum([one] * 3) - np.sum([compute] * 3), 0)
+
+
+# ---- array forms over a whole strategy list ---------------------------------------------------------
+def _hex(x):
+    return float(x).hex()
+
+
+def test_memory_rows_equal_the_class_strategy_by_strategy():
+    """``memory_cost_rows`` (one array evaluation per strategy list, all pipeline stages at once) gives
+    the bits of ``MemoryCostModel`` -- which the recorded reference outputs pin -- for every strategy,
+    stage and the first strategy's 'other' entry, on the seeded memory scenarios."""
+    compared = 0
+    for seed in range(0, C.N_MEMORY, 2):
+        c = C.memory_case(seed)
+        m, t, p, pm, _ = C._records(M, c['prof'], c['model'], c['train'], c['parallel'])
+        rng = np.random.Generator(np.random.PCG64([77, seed]))
+        pp = c['strategy'][0]
+        strs = [c['strategy']] + [s for s in C.all_strategies()
+                                  if s[0] == pp and s[1] % c['kw']['min_tp'] == 0 and rng.random() < 0.5]
+        kw = dict(c['kw'])
+        stages = list(range(pp)) if p.pipeline_type == 'pipedream_flush' else [kw['stage_idx']]
+        kw.pop('stage_idx')
+        rows, other = M.memory_cost_rows(strs, stage_idx=stages, model_args=m, train_args=t, parallel_args=p,
+                                         profile_model_args=pm, **kw)
+        assert rows.shape == (len(stages), len(strs))
+        for j, stage in enumerate(stages):
+            for i, s in enumerate(strs):
+                want = M.MemoryCostModel(s, stage_idx=stage, model_args=m, train_args=t, parallel_args=p,
+                                         profile_model_args=pm, **kw).get_memory_cost()
+                assert _hex(want['enc_total']) == _hex(rows[j, i]), (seed, stage, s)
+                if i == 0 and j == 0:
+                    assert C.jsonable(want['other']) == C.jsonable(other), (seed, s)
+                compared += 1
+        one, _ = M.memory_cost_rows(strs, stage_idx=stages[0], model_args=m, train_args=t, parallel_args=p,
+                                    profile_model_args=pm, **kw)
+        assert one.shape == (len(strs),) and [_hex(x) for x in one] == [_hex(x) for x in rows[0]]
+    assert compared > 2000
+
+
+def test_time_rows_equal_the_class_strategy_by_strategy():
+    compared = 0
+    for seed in range(0, C.N_TIME, 2):
+        c = C.time_case(seed)
+        rng = np.random.Generator(np.random.PCG64([78, seed]))
+        strs = [c['strategy']] + [s for s in C.all_strategies() if rng.random() < 0.3]
+        m, t, p, pm, hw = C._records(M, c['prof'], c['model'], c['train'], c['parallel'])
+        rows = M.time_cost_rows(strs, c['gbsz'], no_comm=c['no_comm'], model_args=m, train_args=t, parallel_args=p,
+                                profile_model_args=pm, profile_hardware_args=hw)
+        assert m.layer_num is not None                    # written back as the class does
+        for i, s in enumerate(strs):
+            m2, t2, p2, pm2, hw2 = C._records(M, c['prof'], c['model'], c['train'], c['parallel'])
+            want = M.TimeCostModel(s, c['gbsz'], no_comm=c['no_comm'], model_args=m2, train_args=t2, parallel_args=p2,
+                                   profile_model_args=pm2, profile_hardware_args=hw2).gen_result()
+            assert _hex(want) == _hex(rows[i]), (seed, s)
+            compared += 1
+    assert compared > 4000
+
+
+def test_array_forms_decline_what_they_do_not_cover():
+    """Inputs on which the class asserts, raises or takes a rare path make the array form raise
+    NotVectorisable (its callers then go strategy by strategy), never return something else."""
+    a = _args()
+    mem = dict(model_args=a['model_args'], train_args=a['train_args'], parallel_args=a['parallel_args'],
+               profile_model_args=a['profile_model_args'])
+    mem['parallel_args'].chunks = 2
+    with pytest.raises(M.NotVectorisable):                # a lane without samples
+        M.memory_cost_rows([[1, 8, 1, {}]], 4, 1, 1, 8, **mem)
+    with pytest.raises(M.NotVectorisable):                # tensor-parallel degree without an activation entry
+        M.memory_cost_rows([[1, 16, 1, {}]], 64, 1, 1, 8, **mem)
+    with pytest.raises(M.NotVectorisable):                # min_tp above the strategy's tp
+        M.memory_cost_rows([[1, 2, 4, {'fsdp': 0, 'tp': 1}]], 64, 1, 4, 8, **mem)
+    with pytest.raises(M.NotVectorisable):                # no layout flag although both tp and dp are above 1
+        M.time_cost_rows([[1, 2, 4, {'fsdp': 0}]], 64, **a)
+    with pytest.raises(M.NotVectorisable):
+        M.time_cost_rows([], 64, **a)
