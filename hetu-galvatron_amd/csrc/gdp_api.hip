@@ -446,6 +446,13 @@ struct gdp_plan {
     int latency_override = -1;  // GALVATRON_DP_LATENCY_VARIANT=0|1|2|4: never / wherever it exists, sources of a
                                 // task on as many waves as the rule says / on 2 / on 4 (tuning aid)
     bool poison = false;     // test aid: NaN-fill the not-yet-written cost buffers before each run
+    // gdp_debug_check_layout: the plan is laid out for a device that is only described (CUs, LDS per CU);
+    // nothing is allocated, uploaded or launched, dbase is an address that is never dereferenced, and the
+    // host copy of the tables always lives in `stage`
+    bool dry = false;
+    size_t small_bytes = 0;  // bytes of the tables at the start of the allocation (what `stage` / lane.up hold)
+    int dry_num_cu = 0;
+    size_t dry_lds_per_cu = 0;
 };
 
 int gdp_validate(const gdp_problem *p, int i)
@@ -536,6 +543,10 @@ int validate(const gdp_problem *p, int i) { return gdp_validate(p, i); }
 void destroy(gdp_plan *pl)
 {
     if (!pl) return;
+    if (pl->dry) {
+        delete pl;
+        return;
+    }
     if (pl->dbase || pl->lane.stream) (void)hipSetDevice(pl->device);
     if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read its host copy
     if (pl->holds_fused) {  // a run that was started and never waited for: its launch has ended by now
@@ -611,7 +622,7 @@ constexpr int GDP_RETRY_WITH_MARKS = 1 << 20;
 int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks)
 {
     pl->n = n;
-    GDP_HIP(hipGetDevice(&pl->device));
+    if (!pl->dry) GDP_HIP(hipGetDevice(&pl->device));
     // defaults of the plan options can be preset from the environment
     bool fused_preset = false;
     if (const char *e = getenv("GALVATRON_DP_FUSED")) {
@@ -651,7 +662,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         fused_preset = true;
     }
     // ---- shapes -------------------------------------------------------------------------------
-    {
+    if (pl->dry) {
+        pl->num_cu = pl->dry_num_cu;
+        pl->lds_per_cu = pl->dry_lds_per_cu;
+    } else {
         hipDeviceProp_t prop;
         GDP_HIP(hipGetDeviceProperties(&prop, pl->device));
         pl->num_cu = prop.multiProcessorCount;
@@ -856,6 +870,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
     }
     const size_t small_bytes = off;
+    pl->small_bytes = small_bytes;
     // words that every fused run resets to zero: completion counters, abort flag
     pl->off_zero = off;
     for (auto &g : pl->groups) {
@@ -886,6 +901,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             h.off_M = pl->keep_marks ? take((size_t)h.L * h.S * (size_t)h.ldm) : 0;
         }
         pl->dbytes = off;
+        if (pl->dry) {
+            pl->dbase = reinterpret_cast<char *>((uintptr_t)1 << 44);  // never dereferenced
+            pl->dalloc = pl->dbytes;
+            break;
+        }
         hipError_t e = arena_take(pl->device, pl->dbytes, &pl->dbase, &pl->dalloc);
         if (e == hipSuccess) break;
         pl->dbase = nullptr;
@@ -902,7 +922,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         return fail_hip(e, buf);
     }
     // ---- build the small region on the host ------------------------------------------------------
-    {
+    if (!pl->dry) {
         const hipError_t e = lane_take(pl->device, pl->back_bytes, small_bytes, &pl->lane);
         if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
             (void)hipGetLastError();
@@ -914,7 +934,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->ev_end = pl->lane.ev_end;
     }
     struct { char *p; char *data() const { return p; } } stage = {pl->lane.up};
-    if (small_bytes > UPLOAD_PINNED_MAX) {
+    if (small_bytes > UPLOAD_PINNED_MAX || pl->dry) {
         try {
             pl->stage.assign(small_bytes, 0);
         } catch (const std::bad_alloc &) {
@@ -1106,6 +1126,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
+    if (pl->dry) {
+        pl->inst.swap(inst);
+        return GDP_OK;
+    }
     GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
@@ -1117,6 +1141,159 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);
+    return GDP_OK;
+}
+
+
+// ---- audit of a laid-out plan (gdp_debug_check_layout) -----------------------------------------------
+// Every address the kernels form from these tables, bounded against the sub-allocation it must stay
+// in.  The bounds restate what the kernels touch:
+//   relaxation (relax_task, relax_task_lat): source elements src + roff[l][s'] + u, u in [0, ntile * tile
+//     rows), s' in [0, SU + GDP_SRC_PAD) (the entries from SU on are the targets of the last prefetches);
+//     transition rows it + s' * SP + column, the same s', columns [0, SP); intra ia + [0, SP);
+//     destination dst + s * ld + u and argmin m + s * ldm + u, s in [0, S), the same u;
+//   fill of the rows below a band: dst-side elements [0, lo * tile rows) of rows [0, S) of buffer l + 1;
+//   fused launches: counters cnt + (instance * max_L + layer) * max_ntile + tile;
+//   epilogue: H + (L % nbuf) * hstride + roff[L][s] + v0 with v0 in [0, V), the argmin table
+//     M + (l * S + s) * ldm + v, v in [0, V), strategy lists res + res_off + [0, L).
+int audit(const gdp_plan *pl, const gdp_problem *const *p)
+{
+    char buf[256];
+    auto bad = [&](const char *what, long long a, long long b, long long c) {
+        snprintf(buf, sizeof buf, "layout audit: %s (%lld, %lld, %lld)", what, a, b, c);
+        return fail(GDP_E_HIP, buf);
+    };
+    const char *stage = pl->stage.data();
+    if (pl->stage.size() < pl->small_bytes) return bad("host copy of the tables is short", (long long)pl->stage.size(), (long long)pl->small_bytes, 0);
+    const uintptr_t base = reinterpret_cast<uintptr_t>(pl->dbase);
+    auto off_of = [&](const void *q) { return (long long)(reinterpret_cast<uintptr_t>(q) - base); };
+    // sub-allocations: inside the allocation and disjoint
+    struct Span { size_t lo, hi; };
+    std::vector<Span> spans;
+    auto span = [&](size_t lo, size_t bytes) { spans.push_back({lo, lo + bytes}); };
+    span(pl->off_insts, sizeof(GdpDevInst) * (size_t)pl->n);
+    span(pl->off_keys, sizeof(GdpDevKey) * (size_t)std::max(pl->n_key_total, 1));
+    span(pl->off_out, sizeof(GdpDevOut) * (size_t)std::max(pl->n_key_total, 1));
+    span(pl->off_res, sizeof(int32_t) * std::max<size_t>(pl->n_res_total, 1));
+    span(pl->off_abort, sizeof(int32_t));
+    for (const Group &g : pl->groups) {
+        span(g.off_active, sizeof(int32_t) * (size_t)g.max_L);
+        span(g.off_lay, sizeof(GdpDevLayer) * (size_t)g.count * (size_t)g.max_L);
+        span(g.off_rows, sizeof(int32_t) * std::max<size_t>(g.rows.size(), 1));
+        span(g.off_cnt, sizeof(int32_t) * (size_t)g.count * g.max_L * g.max_ntile);
+    }
+    for (const HostInst &h : pl->inst) {
+        const size_t rows = (size_t)h.SU + GDP_SRC_PAD;
+        span(h.off_inter, sizeof(double) * (size_t)h.n_inter * rows * h.SP);
+        span(h.off_intra, sizeof(double) * (size_t)h.L * h.SP);
+        span(h.off_index, sizeof(int32_t) * (size_t)h.L);
+        span(h.off_roff, sizeof(int64_t) * (size_t)(h.L + 1) * rows);
+        span(h.off_mem, sizeof(int32_t) * (size_t)h.L * h.S);
+        span(h.off_H, sizeof(double) * (size_t)h.nbuf * (size_t)(h.S + 1) * (size_t)h.ld);
+        if (pl->keep_marks) span(h.off_M, (size_t)h.L * h.S * (size_t)h.ldm);
+    }
+    std::sort(spans.begin(), spans.end(), [](const Span &a, const Span &b) { return a.lo < b.lo; });
+    for (size_t i = 0; i < spans.size(); ++i) {
+        if (spans[i].hi > pl->dbytes) return bad("sub-allocation beyond the allocation", (long long)spans[i].lo, (long long)spans[i].hi, (long long)pl->dbytes);
+        if (i && spans[i].lo < spans[i - 1].hi) return bad("sub-allocations overlap", (long long)spans[i - 1].lo, (long long)spans[i - 1].hi, (long long)spans[i].lo);
+    }
+    const GdpDevInst *di = reinterpret_cast<const GdpDevInst *>(stage + pl->off_insts);
+    const GdpDevKey *dk = reinterpret_cast<const GdpDevKey *>(stage + pl->off_keys);
+    for (int i = 0; i < pl->n; ++i) {
+        const HostInst &h = pl->inst[(size_t)i];
+        const gdp_problem *q = p[h.orig];
+        const GdpDevInst &d = di[i];
+        const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
+        const long long rows = (long long)h.SU + GDP_SRC_PAD;
+        const long long span_u = (long long)h.ntile * tile_rows;      // source rows a launch touches
+        const long long buf_elems = (long long)(h.S + 1) * h.ld;
+        if (h.SP % GDP_VARIANTS[h.variant].ts || h.SP < h.S || h.SU < h.S) return bad("strategy padding", h.SP, h.SU, h.S);
+        if (span_u < h.V || h.ldm < span_u || h.ld < h.P + span_u) return bad("row length", h.ld, h.ldm, span_u);
+        if (off_of(d.H) != (long long)h.off_H || d.hstride != buf_elems || d.nbuf != h.nbuf || h.nbuf < 2)
+            return bad("cost buffers of the instance record", off_of(d.H), d.hstride, d.nbuf);
+        if (off_of(d.inter) != (long long)h.off_inter || off_of(d.intra) != (long long)h.off_intra ||
+            off_of(d.inter_index) != (long long)h.off_index || off_of(d.roff) != (long long)h.off_roff ||
+            off_of(d.mem) != (long long)h.off_mem || (pl->keep_marks && off_of(d.M) != (long long)h.off_M))
+            return bad("table pointers of the instance record", i, 0, 0);
+        // row offsets: every source element a task or the epilogue can form stays inside one cost buffer
+        const int64_t *ro = reinterpret_cast<const int64_t *>(stage + h.off_roff);
+        for (int l = 0; l <= h.L; ++l)
+            for (long long s = 0; s < rows; ++s) {
+                const long long o = ro[(size_t)l * rows + s];
+                if (o < 0 || o + span_u > buf_elems) return bad("row offset leaves the cost buffer", l, s, o);
+                // a real strategy reads its own row shifted down by its memory cost, or the +inf row
+                if (s < h.S && l > 0) {
+                    const int m = q->mem[(size_t)(l - 1) * h.S + s];
+                    const long long want = m >= h.V ? (long long)h.S * h.ld + h.P : s * h.ld + h.P - m;
+                    if (o != want || (m < h.V && m > h.P)) return bad("row offset of a strategy", l, s, o);
+                }
+            }
+        const int32_t *ix = reinterpret_cast<const int32_t *>(stage + h.off_index);
+        for (int l = 0; l < h.L; ++l)
+            if (ix[l] < 0 || ix[l] >= h.n_inter) return bad("transition-matrix index", l, ix[l], h.n_inter);
+        for (int k = 0; k < h.n_key; ++k) {
+            const GdpDevKey &key = dk[h.key_begin + k];
+            if (key.inst != i) return bad("instance of a key", i, k, key.inst);
+            if (key.res_off < 0 || (size_t)key.res_off + (size_t)h.L > pl->n_res_total) return bad("strategy list of a key", i, k, key.res_off);
+            if (key.other_mem < 0) return bad("start row above the table", i, k, (long long)key.other_mem);
+        }
+    }
+    for (const Group &g : pl->groups) {
+        const GdpDevLayer *lay = reinterpret_cast<const GdpDevLayer *>(stage + g.off_lay);
+        const int tile_rows = 64 * GDP_VARIANTS[g.variant].r;
+        if (g.ntb * GDP_VARIANTS[g.variant].ts != g.SP) return bad("target blocks of a group", g.ntb, g.SP, 0);
+        if (off_of(g.sched.lay) != (long long)g.off_lay || off_of(g.sched.cnt) != (long long)g.off_cnt ||
+            off_of(g.sched.n_active) != (long long)g.off_active || off_of(g.sched.abort_flag) != (long long)pl->off_abort ||
+            g.sched.max_L != g.max_L || g.sched.max_ntile != g.max_ntile)
+            return bad("launch record of a group", g.first, 0, 0);
+        for (int k = 0; k < g.count; ++k) {
+            const HostInst &h = pl->inst[(size_t)(g.first + k)];
+            const long long rows = (long long)h.SU + GDP_SRC_PAD;
+            if (h.ntile > g.max_ntile || h.L > g.max_L || h.SP != g.SP) return bad("instance against its group", k, h.ntile, h.L);
+            for (int l = 0; l < g.max_L; ++l) {
+                const GdpDevLayer &y = lay[(size_t)k * g.max_L + l];
+                if (l >= h.L) {
+                    if (y.hi >= y.lo) return bad("a layer the instance does not have is not empty", k, l, y.hi);
+                    continue;
+                }
+                const long long H0 = (long long)h.off_H, buf_bytes = (long long)sizeof(double) * (h.S + 1) * h.ld;
+                const long long src = off_of(y.src) - H0, dst = off_of(y.dst) - H0 - (long long)sizeof(double) * h.P;
+                if (src < 0 || src % buf_bytes || src / buf_bytes >= h.nbuf) return bad("source buffer of a layer", k, l, src);
+                if (dst < 0 || dst % buf_bytes || dst / buf_bytes >= h.nbuf || dst == src) return bad("destination buffer of a layer", k, l, dst);
+                if (src / buf_bytes != l % h.nbuf || dst / buf_bytes != (l + 1) % h.nbuf) return bad("buffer order of a layer", k, l, 0);
+                if (off_of(y.ro) != (long long)h.off_roff + (long long)sizeof(int64_t) * l * rows) return bad("row offsets of a layer", k, l, 0);
+                const long long mat = (off_of(y.it) - (long long)h.off_inter) / ((long long)sizeof(double) * rows * h.SP);
+                if (off_of(y.it) != (long long)h.off_inter + mat * (long long)sizeof(double) * rows * h.SP || mat < 0 || mat >= h.n_inter)
+                    return bad("transition matrix of a layer", k, l, mat);
+                if (off_of(y.ia) != (long long)h.off_intra + (long long)sizeof(double) * l * h.SP) return bad("intra row of a layer", k, l, 0);
+                if (pl->keep_marks ? off_of(y.m) != (long long)h.off_M + (long long)l * h.S * h.ldm : y.m != nullptr)
+                    return bad("argmin rows of a layer", k, l, 0);
+                if (y.ld != h.ld || y.ldm != h.ldm || y.S != h.S || y.SU != h.SU || y.SP != h.SP || y.ntile != h.ntile)
+                    return bad("shape fields of a layer", k, l, 0);
+                if (y.lo < 0 || y.lo > h.ntile || y.hi < -1 || y.hi >= h.ntile || y.dep < 0) return bad("band of a layer", y.lo, y.hi, y.dep);
+                if ((long long)y.lo * tile_rows > h.ldm) return bad("filled rows beyond a row", k, l, y.lo);
+            }
+        }
+        for (size_t r = 0; r + 2 < g.rows.size(); r += 3) {
+            const int first = g.rows[r], cnt = g.rows[r + 1], layer = g.rows[r + 2];
+            if (first < 0 || cnt < 1 || first + cnt > g.count || layer < 0 || layer >= pl->inst[(size_t)(g.first + first)].L)
+                return bad("row of a chunked launch", first, cnt, layer);
+        }
+        for (const auto &seg : g.segments) {
+            const long long rows_total = g.rows.empty() ? g.max_L : (long long)(g.rows.size() / 3);
+            if (seg.first < 0 || seg.layers < 1 || seg.layers > 65535 || seg.first + seg.layers > rows_total)
+                return bad("segment of fused launches", seg.first, seg.layers, rows_total);
+            const long long grid_x = 8LL * (g.rows.empty() ? g.active[(size_t)seg.first] : g.chunk) * g.slots;
+            if (grid_x < 1 || grid_x > 0x7fffffffLL || g.slots < 1) return bad("grid of a fused launch", grid_x, g.slots, 0);
+            if (seg.lds_bytes > 65536u) return bad("dynamic LDS of a fused launch", seg.lds_bytes, 0, 0);
+        }
+        const long long tasks = (long long)g.max_ntile * g.ntb * (g.latency > 1 ? g.latency : 1);
+        if (tasks / GDP_WAVES_PER_BLOCK + 16 > 0x7fffffffLL || g.count > 65535) return bad("grid of a per-layer launch", tasks, g.count, 0);
+        if (g.latency && (g.latency != 1 && g.latency != 2 && g.latency != 4)) return bad("latency variant", g.latency, 0, 0);
+        if (g.latency)
+            for (int k = 0; k < g.count; ++k)
+                if (pl->inst[(size_t)(g.first + k)].SU % (GDP_SRC_UNROLL_LAT * g.latency)) return bad("source padding of the latency variant", k, g.latency, 0);
+    }
     return GDP_OK;
 }
 
@@ -1385,6 +1562,38 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
 }
 
 void gdp_plan_destroy(gdp_plan *plan) { destroy(plan); }
+
+int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_cu, int64_t lds_per_cu)
+{
+    gdp_clear_error();
+    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
+    if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
+    if (num_cu < 1 || lds_per_cu < 0) return fail(GDP_E_BADARG, "bad device description");
+    for (int i = 0; i < n; ++i) {
+        const int rc = validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+    }
+    for (int attempt = 0; attempt < 2; ++attempt) {     // costs only first, then with the argmin table where S allows
+        gdp_plan *pl = new (std::nothrow) gdp_plan();
+        if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
+        pl->dry = true;
+        pl->dry_num_cu = num_cu;
+        pl->dry_lds_per_cu = (size_t)lds_per_cu;
+        int rc;
+        try {
+            rc = create(n, p, pl, attempt == 1);
+            if (rc == GDP_OK) rc = audit(pl, p);
+        } catch (const std::bad_alloc &) {
+            rc = fail(GDP_E_NOMEM, "host allocation failed");
+        }
+        destroy(pl);
+        if (rc != GDP_OK) return rc;
+        bool marks_possible = true;
+        for (int i = 0; i < n; ++i) marks_possible = marks_possible && p[i]->S <= GDP_MAX_S_MARKS;
+        if (!marks_possible) break;
+    }
+    return GDP_OK;
+}
 
 void gdp_cache_trim(void)
 {

@@ -38,7 +38,7 @@ GDP_STATIC_SCRATCH_BYTES = 64 << 20
 
 EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_solve_static", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
                     "gdp_plan_destroy", "gdp_plan_set_option", "gdp_cache_trim", "gdp_last_error", "gdp_version",
-                    "gdp_device_info")
+                    "gdp_device_info", "gdp_debug_check_layout")
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -110,6 +110,8 @@ def lib() -> ctypes.CDLL:
         L.gdp_version.restype = ctypes.c_int
         L.gdp_device_info.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
         L.gdp_device_info.restype = ctypes.c_int
+        L.gdp_debug_check_layout.argtypes = [ctypes.c_int32, pp, ctypes.c_int32, ctypes.c_int64]
+        L.gdp_debug_check_layout.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -208,6 +210,13 @@ def solve_batch(problems: Sequence[Problem]) -> None:
         return
     P, R = _arrays(problems)
     _check(lib().gdp_solve_batch(len(problems), P, R))
+
+
+def check_layout(problems: Sequence[Problem], num_cu: int = 256, lds_per_cu: int = 160 * 1024) -> None:
+    """gdp_debug_check_layout: lays the plan out for a described device (no device needed) and checks
+    every address the kernels would form; raises with the violated bound."""
+    P, _ = _arrays(problems)
+    _check(lib().gdp_debug_check_layout(len(problems), P, num_cu, lds_per_cu))
 
 
 def solve_static(problem: Problem) -> None:

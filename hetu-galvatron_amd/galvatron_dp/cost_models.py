@@ -846,7 +846,9 @@ def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_arg
                       profile_model_args=profile_model_args_list[t],
                       profile_hardware_args=profile_hardware_args_list[t])
         rows = None
-        if timecostmodel is TimeCostModel:              # this package's own model: all strategies at once
+        # this package's own model: all strategies at once -- where there are enough of them for one array
+        # evaluation (some sixty array operations) to be cheaper than an object per strategy
+        if timecostmodel is TimeCostModel and len(texts) >= 8:
             try:
                 parsed = [strategy_str2list(text) for text in texts]
                 rows = (time_cost_rows(parsed, bsz_per_chunk[t], **common),

@@ -177,6 +177,15 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
  * and destroying a stream takes a third as long as a small solve); this call releases those too. */
 void gdp_cache_trim(void);
 
+/* Test aid (no counterpart in the reference): validates the problems, lays a plan out exactly as
+ * gdp_plan_create would for a device with num_cu compute units and lds_per_cu bytes of LDS per unit --
+ * once in the default layout and once in the one that keeps the argmin table -- and checks every
+ * address the kernels would form from the resulting tables against the sub-allocation it must stay
+ * in.  Needs no device: nothing is allocated, uploaded or launched.  GDP_OK, a validation error, or
+ * GDP_E_HIP with the violated bound in gdp_last_error().  The plan options that can be preset from the
+ * environment (GALVATRON_DP_FUSED, _SKIP, _TILE_TS, _TILE_R, _CHUNK, _LATENCY_VARIANT ...) apply. */
+int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_cu, int64_t lds_per_cu);
+
 /* Text of the calling thread's last error ("" if none). */
 const char *gdp_last_error(void);
 /* GDP_VERSION of the built library. */
