@@ -318,6 +318,8 @@ struct HostInst {
     int res_begin;  // first element in the result array
     // byte offsets inside the device allocation
     size_t off_H, off_M, off_inter, off_intra, off_index, off_roff, off_mem;
+    bool has_zero = false;  // some memory cost is 0 (see gdp_launch_zero_pass)
+    size_t off_zcols = 0;
 };
 
 struct Group {  // instances with the same S, sorted by L descending
@@ -330,6 +332,8 @@ struct Group {  // instances with the same S, sorted by L descending
     struct Segment { int first, layers; unsigned lds_bytes; };
     std::vector<Segment> segments;  // fused launches: runs of layers with the same active set, or -- chunked --
                                     // runs of at most 65535 entries of the row table
+    std::vector<char> zero_layer;   // [max_L] some instance of the group has a strategy with mem == 0 in layer l
+    int max_V = 0;
     int latency = 0;                // per-layer launches use the variant for launches with few waves: 0, or the
                                     // number of waves (1, 2, 4) that share the source strategies of a task
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
@@ -449,6 +453,8 @@ struct gdp_plan {
     // gdp_debug_check_layout: the plan is laid out for a device that is only described (CUs, LDS per CU);
     // nothing is allocated, uploaded or launched, dbase is an address that is never dereferenced, and the
     // host copy of the tables always lives in `stage`
+    bool has_zero = false;   // some instance has a memory cost of 0: one launch per layer, each followed by the
+                             // pass that redoes those strategies in the reference's in-place order
     bool dry = false;
     size_t small_bytes = 0;  // bytes of the tables at the start of the allocation (what `stage` / lane.up hold)
     int dry_num_cu = 0;
@@ -477,8 +483,6 @@ int gdp_validate(const gdp_problem *p, int i)
     const size_t LS = (size_t)p->L * p->S;
     for (size_t k = 0; k < LS; ++k) {
         if (p->mem[k] < 0) return bad(GDP_E_BADARG, "negative mem entry");
-        if (p->mem[k] == 0)
-            return bad(GDP_E_UNSUPPORTED, "mem entry equal to 0 (in-place update reads its own row)");
     }
     if (p->inter_index)
         for (int l = 0; l < p->L; ++l)
@@ -656,10 +660,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         if (p[i]->flags & GDP_LAUNCH_FUSED) { pl->fused = true; fused_preset = true; }
         else if (p[i]->flags & GDP_LAUNCH_PER_LAYER) { pl->fused = false; fused_preset = true; }
     }
-    if (force_marks) {
-        pl->keep_marks = true;
-        pl->fused = false;
-        fused_preset = true;
+    for (int i = 0; i < n && !pl->has_zero; ++i)
+        for (size_t k = 0; k < (size_t)p[i]->L * p[i]->S; ++k)
+            if (p[i]->mem[k] == 0) {
+                pl->has_zero = true;
+                break;
+            }
+    if (force_marks || pl->has_zero) {
+        if (force_marks) pl->keep_marks = true;
+        pl->fused = false;    // (mem == 0: a cell then depends on cells of its own layer, which the counters of a
+        fused_preset = true;  //  fused launch do not order)
     }
     // ---- shapes -------------------------------------------------------------------------------
     if (pl->dry) {
@@ -682,8 +692,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.n_inter = q->inter_index ? q->n_inter : q->L;
         h.flags = q->flags;
         int maxm = 0;
-        for (size_t k = 0; k < (size_t)q->L * q->S; ++k)
+        for (size_t k = 0; k < (size_t)q->L * q->S; ++k) {
             if (q->mem[k] < q->V) maxm = std::max(maxm, q->mem[k]);
+            if (q->mem[k] == 0) h.has_zero = true;
+        }
         h.P = (int)align_up((size_t)std::max(maxm, 1), 64);
     }
     // group by S, then by L descending (stable, so equal shapes keep the caller's order)
@@ -763,8 +775,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             g.max_ld = std::max(g.max_ld, h.ld);
         }
         g.active.assign((size_t)g.max_L, 0);
-        for (int k = i; k < j; ++k)
-            for (int l = 0; l < inst[(size_t)k].L; ++l) g.active[(size_t)l]++;
+        g.zero_layer.assign((size_t)g.max_L, 0);
+        for (int k = i; k < j; ++k) {
+            g.max_V = std::max(g.max_V, inst[(size_t)k].V);
+            for (int l = 0; l < inst[(size_t)k].L; ++l) {
+                g.active[(size_t)l]++;
+                if (inst[(size_t)k].has_zero)
+                    for (int s2 = 0; s2 < g.S; ++s2)
+                        if (p[inst[(size_t)k].orig]->mem[(size_t)l * g.S + s2] == 0) g.zero_layer[(size_t)l] = 1;
+            }
+        }
         g.nbt = (g.max_ntile * g.ntb + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK;
         // Whole tiles per XCD turn: the fewest whose wave tasks fill whole workgroups.  (Longer turns
         // would save some of the cache lines that neighbouring tiles share -- a tile's source rows start
@@ -868,6 +888,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
         h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_PAD));
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
+        h.off_zcols = h.has_zero ? take(sizeof(int32_t) * (size_t)h.L * (size_t)(h.S + 1)) : 0;
     }
     const size_t small_bytes = off;
     pl->small_bytes = small_bytes;
@@ -892,10 +913,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         return fail(GDP_E_BADARG, "S exceeds GDP_MAX_S_MARKS and the argmin table is to be kept");
     for (int attempt = 0; attempt < 2; ++attempt) {
         off = fixed_bytes;
-        pl->can_fuse = pl->fused || !pl->keep_marks;
+        pl->can_fuse = (pl->fused || !pl->keep_marks) && !pl->has_zero;
         pl->rezero = false;
         for (auto &h : inst) {
-            h.nbuf = pl->can_fuse ? h.L + 1 : 2;
+            h.nbuf = (pl->can_fuse || !pl->keep_marks) ? h.L + 1 : 2;   // costs only: the backtrack needs every layer's costs
             if (h.nbuf < h.L + 1) pl->rezero = true;
             h.off_H = take(sizeof(double) * (size_t)h.nbuf * (size_t)(h.S + 1) * (size_t)h.ld);
             h.off_M = pl->keep_marks ? take((size_t)h.L * h.S * (size_t)h.ldm) : 0;
@@ -910,8 +931,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         if (e == hipSuccess) break;
         pl->dbase = nullptr;
         (void)hipGetLastError();
-        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && !pl->keep_marks &&
-            max_S <= GDP_MAX_S_MARKS)
+        if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && !pl->keep_marks && max_S <= GDP_MAX_S_MARKS)
             return GDP_RETRY_WITH_MARKS;  // tile widths and paddings differ with the table: start over
         if ((e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) && pl->can_fuse && pl->keep_marks) {
             pl->fused = false;            // table kept and all layers in one launch: drop the latter
@@ -978,6 +998,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         int32_t *ix = reinterpret_cast<int32_t *>(stage.data() + h.off_index);
         for (int l = 0; l < h.L; ++l) ix[l] = q->inter_index ? q->inter_index[l] : l;
         memcpy(stage.data() + h.off_mem, q->mem, sizeof(int32_t) * (size_t)h.L * h.S);
+        d.zcols = nullptr;
+        if (h.has_zero) {
+            d.zcols = reinterpret_cast<const int32_t *>(pl->dbase + h.off_zcols);
+            int32_t *z = reinterpret_cast<int32_t *>(stage.data() + h.off_zcols);
+            for (int l = 0; l < h.L; ++l) {
+                int32_t *row = z + (size_t)l * (h.S + 1);
+                row[0] = 0;
+                for (int s = 0; s < h.S; ++s)
+                    if (q->mem[(size_t)l * h.S + s] == 0) row[++row[0]] = s;
+            }
+        }
         // roff[l][s']: where row 0 of "f after layer l-1, strategy s'" sits in a cost buffer
         int64_t *ro = reinterpret_cast<int64_t *>(stage.data() + h.off_roff);
         const int64_t inf_row = (int64_t)h.S * h.ld + h.P;
@@ -1189,6 +1220,7 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
         span(h.off_index, sizeof(int32_t) * (size_t)h.L);
         span(h.off_roff, sizeof(int64_t) * (size_t)(h.L + 1) * rows);
         span(h.off_mem, sizeof(int32_t) * (size_t)h.L * h.S);
+        if (h.has_zero) span(h.off_zcols, sizeof(int32_t) * (size_t)h.L * (size_t)(h.S + 1));
         span(h.off_H, sizeof(double) * (size_t)h.nbuf * (size_t)(h.S + 1) * (size_t)h.ld);
         if (pl->keep_marks) span(h.off_M, (size_t)h.L * h.S * (size_t)h.ldm);
     }
@@ -1352,6 +1384,8 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                 GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, pl->keep_marks ? 0 : g.latency,
                                          reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
                                          g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
+                if (g.zero_layer[(size_t)l])
+                    GDP_HIP(gdp_launch_zero_pass(pl->keep_marks, d_insts + g.first, g.active[(size_t)l], g.max_V, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
@@ -1540,7 +1574,7 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
     switch (option) {
         case GDP_OPT_FUSED:
             if (value != 0 && !plan->can_fuse)
-                return fail(GDP_E_BADARG, "plan was laid out with two cost buffers (per-layer launches only)");
+                return fail(GDP_E_BADARG, "plan was laid out for per-layer launches only (two cost buffers, or a memory cost of 0)");
             plan->fused = value != 0;
             return GDP_OK;
         case GDP_OPT_POISON:

@@ -56,6 +56,7 @@ struct GdpDevInst {
     const int32_t *inter_index;
     const int64_t *roff;
     const int32_t *mem;
+    const int32_t *zcols;   // null, or L rows of S+1 int32: {n, the n strategies of the layer whose memory cost is 0, ascending}
     int64_t ld;          // elements per row of H
     int64_t ldm;         // entries per row of M
     int32_t L, V, S, SP;
@@ -159,6 +160,15 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
                            int max_L, int tile_rows, int what, hipStream_t stream);
 // Fills n int32 with zero (queue counters; a kernel rather than a memset so that it can be captured).
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream);
+// Strategies whose memory cost is 0 in layer `layer`, for the first n_inst instances (those that have
+// such a layer and such strategies; the others are skipped).  The reference updates f in place, bin v
+// downwards and strategy s upwards (csrc/dp_core.cpp:58-73): a cell with mem == 0 reads its OWN row,
+// where the entries of lower strategies already hold this layer's values.  After the layer's ordinary
+// launch (which has given every strategy with mem > 0 its final value, from the previous layer's
+// buffer alone) this pass recomputes the mem == 0 columns, one lane per bin, in ascending strategy
+// order: candidates from lower strategies come from the buffer the layer writes, the others from the
+// buffer it reads.  One launch per layer only (plans with such strategies never fuse layers).
+hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, int n_inst, int max_V, int layer, hipStream_t stream);
 // argmin over the last layer's row + backtrack, one wavefront per key (marks: through the stored
 // argmin table; otherwise recomputed from the cost buffers of all layers).
 hipError_t gdp_launch_epilogue(bool marks, const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,

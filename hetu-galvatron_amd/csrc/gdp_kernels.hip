@@ -718,6 +718,56 @@ __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restr
     }
 }
 
+// ---- strategies with a memory cost of 0 -------------------------------------------------------------
+// See gdp_launch_zero_pass.  grid = (blocks of 256 bins, instances).  A lane owns bin v and walks the
+// layer's mem == 0 strategies in ascending order; what it stores for one of them is what it (and only
+// it) reads back as a candidate of the next ones.  Candidates, association and tie-break are the
+// reference's: (f + inter) + intra, ascending source strategies, replaced on strict '<'
+// (csrc/dp_core.cpp:65-72).
+template <bool MARKS>
+__global__ __launch_bounds__(256) void gdp_zero_pass_kernel(const GdpDevInst *insts, int layer)
+{
+    const GdpDevInst *I = insts + blockIdx.y;
+    const int32_t *zc = uload(&I->zcols);
+    if (!zc || layer >= uload(&I->L)) return;
+    const int S = uload(&I->S), V = uload(&I->V);
+    const int32_t *z = zc + (int64_t)layer * (S + 1);
+    const int nz = uload(z);
+    const int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (nz == 0 || v >= V) return;
+    const int rows = uload(&I->SU) + GDP_SRC_PAD, SP = uload(&I->SP), nbuf = uload(&I->nbuf);
+    const int64_t hstride = uload(&I->hstride);
+    double *H = uload(&I->H);
+    const double *old_costs = H + (int64_t)(layer % nbuf) * hstride;      // what the layer reads
+    double *new_costs = H + (int64_t)((layer + 1) % nbuf) * hstride;      // what it writes
+    const int64_t *ro_old = uload(&I->roff) + (int64_t)layer * rows;
+    const int64_t *ro_new = ro_old + rows;
+    const double *it = uload(&I->inter) + (int64_t)uload(uload(&I->inter_index) + layer) * rows * SP;
+    const double *ia = uload(&I->intra) + (int64_t)layer * SP;
+    [[maybe_unused]] uint8_t *M = nullptr;
+    [[maybe_unused]] int64_t ldm = 0;
+    if constexpr (MARKS) {
+        ldm = uload(&I->ldm);
+        M = uload(&I->M) + (int64_t)layer * S * ldm;
+    }
+    for (int k = 0; k < nz; ++k) {
+        const int s = uload(z + 1 + k);
+        const double a = uload(ia + s);
+        double best = 0;
+        int arg = 0;
+        for (int sp = 0; sp < S; ++sp) {
+            const double x = sp < s ? new_costs[uload(ro_new + sp) + v] : old_costs[uload(ro_old + sp) + v];
+            const double c = (x + uload(it + (int64_t)sp * SP + s)) + a;
+            if (sp == 0 || c < best) {
+                best = c;
+                arg = sp;
+            }
+        }
+        new_costs[uload(ro_new + s) + v] = best;     // mem == 0: the cell's own bin
+        if constexpr (MARKS) M[(int64_t)s * ldm + v] = (uint8_t)arg;
+    }
+}
+
 // ---- wavefront (value, index) reduction: lower value wins, equal values -> lower index ----------
 __device__ __forceinline__ double swz_f64(double x, int pattern_sel)
 {
@@ -847,7 +897,8 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
                     a_next = intra[(int64_t)(i - 1) * SP + sl];
                     t_next = uload(inter_index + (i - 1));
                 }
-                v -= __builtin_amdgcn_readlane(m_cur, cur);  // the source row of cell (i, v, cur)
+                const int m_here = __builtin_amdgcn_readlane(m_cur, cur);
+                v -= m_here;  // the source row of cell (i, v, cur)
                 if (v < 0) break;
                 const double *src = H + (int64_t)(i % nbuf) * hstride;  // costs before layer i
                 const double a = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(a_cur), cur),
@@ -855,7 +906,11 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
                 double bv = INFINITY;
                 int bi = 0x7fffffff;
                 if (lane < S) {
-                    bv = (src[r_cur + v] + inter[((int64_t)t_cur * rows + lane) * SP + cur]) + a;
+                    // a cell with mem == 0 took its lower strategies from its own layer (gdp_launch_zero_pass)
+                    const double x = (m_here == 0 && lane < cur)
+                                         ? H[(int64_t)((i + 1) % nbuf) * hstride + roff[(int64_t)(i + 1) * rows + lane] + v]
+                                         : src[r_cur + v];
+                    bv = (x + inter[((int64_t)t_cur * rows + lane) * SP + cur]) + a;
                     bi = lane;
                 }
                 wave_argmin(bv, bi);
@@ -867,16 +922,19 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
         }
         for (; i > 0; --i) {
             const int cur = idx;
-            v -= uload(mem + (int64_t)i * S + cur);  // the source row of cell (i, v, cur)
+            const int m_here = uload(mem + (int64_t)i * S + cur);
+            v -= m_here;  // the source row of cell (i, v, cur)
             if (v < 0) break;
             const double *src = H + (int64_t)(i % nbuf) * hstride;  // costs before layer i
+            const double *own = H + (int64_t)((i + 1) % nbuf) * hstride;  // costs after it
             const int64_t *rl = roff + (int64_t)i * rows;
             const double *it = inter + (int64_t)uload(inter_index + i) * rows * SP + cur;
             const double a = uload(intra + (int64_t)i * SP + cur);
             double bv = INFINITY;
             int bi = 0x7fffffff;
             for (int s = lane; s < S; s += 64) {
-                const double c = (src[rl[s] + v] + it[(int64_t)s * SP]) + a;
+                const double x = (m_here == 0 && s < cur) ? own[rl[rows + s] + v] : src[rl[s] + v];
+                const double c = (x + it[(int64_t)s * SP]) + a;
                 if (c < bv || bi == 0x7fffffff) { bv = c; bi = s; }
             }
             wave_argmin(bv, bi);
@@ -1039,6 +1097,17 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
                                insts + i0, lay + (int64_t)i0 * max_L, max_L, tile_rows);
         }
     }
+    return hipGetLastError();
+}
+
+hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, int n_inst, int max_V, int layer, hipStream_t stream)
+{
+    if (n_inst <= 0 || max_V <= 0) return hipSuccess;
+    dim3 grid((unsigned)((max_V + 255) / 256), (unsigned)n_inst), block(256);
+    if (marks)
+        hipLaunchKernelGGL(gdp_zero_pass_kernel<true>, grid, block, 0, stream, insts, layer);
+    else
+        hipLaunchKernelGGL(gdp_zero_pass_kernel<false>, grid, block, 0, stream, insts, layer);
     return hipGetLastError();
 }
 

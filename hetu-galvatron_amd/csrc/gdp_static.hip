@@ -63,7 +63,8 @@ int scratch_of_device(unsigned char **out)
 struct Layout {
     int L, V, S, T, n_key, ts, variant, SP, SU, rows, P, ntile;
     int64_t ld, ldm;
-    size_t off_inst, off_keys, off_lay, off_inter, off_intra, off_index, off_roff, off_mem, small_bytes;
+    size_t off_inst, off_keys, off_lay, off_inter, off_intra, off_index, off_roff, off_mem, off_zcols, small_bytes;
+    bool has_zero;
     size_t off_out, off_res, back_bytes, off_H, off_M, total_bytes;
 };
 
@@ -83,8 +84,11 @@ void lay_out(const gdp_problem *p, Layout *y)
     y->SU = (int)align_up((size_t)p->S, GDP_SRC_UNROLL);
     y->rows = y->SU + GDP_SRC_PAD;
     int maxm = 1;
-    for (size_t k = 0; k < (size_t)p->L * p->S; ++k)
+    y->has_zero = false;
+    for (size_t k = 0; k < (size_t)p->L * p->S; ++k) {
         if (p->mem[k] < p->V) maxm = std::max(maxm, p->mem[k]);
+        if (p->mem[k] == 0) y->has_zero = true;
+    }
     y->P = (int)align_up((size_t)maxm, 64);
     y->ntile = (p->V + 63) / 64;
     y->ldm = (int64_t)align_up((size_t)y->ntile * 64, 256);
@@ -103,6 +107,7 @@ void lay_out(const gdp_problem *p, Layout *y)
     y->off_index = take(sizeof(int32_t) * (size_t)y->L);
     y->off_roff = take(sizeof(int64_t) * (size_t)(y->L + 1) * y->rows);
     y->off_mem = take(sizeof(int32_t) * (size_t)y->L * y->S);
+    y->off_zcols = y->has_zero ? take(sizeof(int32_t) * (size_t)y->L * (size_t)(y->S + 1)) : 0;
     y->small_bytes = off;
     y->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(y->n_key, 1));
     y->off_res = take(sizeof(int32_t) * std::max<size_t>((size_t)y->n_key * y->L, 1));
@@ -139,6 +144,17 @@ void build(const gdp_problem *p, const Layout &y, unsigned char *base)
     int32_t *ix = reinterpret_cast<int32_t *>(g_stage + y.off_index);
     for (int l = 0; l < y.L; ++l) ix[l] = p->inter_index ? p->inter_index[l] : l;
     memcpy(g_stage + y.off_mem, p->mem, sizeof(int32_t) * (size_t)y.L * y.S);
+    d.zcols = nullptr;
+    if (y.has_zero) {   // per layer: {n, the n strategies whose memory cost is 0} (see gdp_launch_zero_pass)
+        d.zcols = reinterpret_cast<const int32_t *>(base + y.off_zcols);
+        int32_t *z = reinterpret_cast<int32_t *>(g_stage + y.off_zcols);
+        for (int l = 0; l < y.L; ++l) {
+            int32_t *row = z + (size_t)l * (y.S + 1);
+            row[0] = 0;
+            for (int s = 0; s < y.S; ++s)
+                if (p->mem[(size_t)l * y.S + s] == 0) row[++row[0]] = s;
+        }
+    }
     // roff[l][s']: element offset, from the base of a cost buffer, of "f after layer l-1, strategy s', row 0";
     // a strategy whose memory cost reaches V, and every padding source, reads the +inf row
     int64_t *ro = reinterpret_cast<int64_t *>(g_stage + y.off_roff);
@@ -221,8 +237,10 @@ extern "C" int gdp_solve_static(const gdp_problem *p, gdp_result *r)
     // +inf pads and +inf row of both cost buffers, zeros in the first one (the caller's initial f): whatever
     // the last call left there is overwritten before anything reads it
     e = gdp_launch_init(d_inst, 1, y.ld, y.S, d_lay, y.L, 64, GDP_INIT_PADS | GDP_INIT_ZERO, stream);
-    for (int l = 0; l < y.L && e == hipSuccess; ++l)
+    for (int l = 0; l < y.L && e == hipSuccess; ++l) {
         e = gdp_launch_relax(y.variant, true, 0, d_lay, y.L, 1, y.ntile, y.SP, l, stream);
+        if (e == hipSuccess && y.has_zero) e = gdp_launch_zero_pass(true, d_inst, 1, y.V, l, stream);
+    }
     if (e == hipSuccess)
         e = gdp_launch_epilogue(true, d_inst, reinterpret_cast<const GdpDevKey *>(base + y.off_keys), y.n_key,
                                 reinterpret_cast<GdpDevOut *>(base + y.off_out),

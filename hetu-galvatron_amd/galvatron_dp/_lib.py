@@ -46,7 +46,8 @@ _f64p = ctypes.POINTER(ctypes.c_double)
 
 
 class UnsupportedInputError(ValueError):
-    """Input outside what the device recurrence covers (a memory cost of 0)."""
+    """GDP_E_UNSUPPORTED.  No input is answered with it any more (a memory cost of 0, once refused, is
+    computed with the reference's in-place order); kept so that callers catching it keep working."""
 
 
 # The pointer members are declared as untyped pointers (same layout as the typed ones of the header):

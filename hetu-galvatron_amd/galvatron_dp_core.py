@@ -10,8 +10,10 @@ libgalvatron_dp_hip.so; nothing else in the caller changes.
 Differences from the compiled reference module, all on arguments no caller reads back:
 ``_mark`` and ``_f`` are filled only after ``set_export(True)`` (the argmin table lives on the
 device in a compact form, and copying L*V*S int32 back per call would dominate the run time).
-Inputs the device recurrence does not cover raise instead of computing something: NaN / -inf
-costs (``ValueError``) and a memory cost of 0 (``UnsupportedInputError``, a ``ValueError``).
+Inputs on which the reference's result depends on evaluation order or is undefined raise
+``ValueError`` instead of computing something: NaN / -inf costs, negative memory costs, a negative
+``other_mem_cost`` (start row above the table).  A memory cost of 0 is computed with the reference's
+in-place order (csrc/dp_core.cpp:58-73).
 """
 from __future__ import annotations
 

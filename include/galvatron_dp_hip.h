@@ -35,7 +35,7 @@ extern "C" {
 /* return codes */
 #define GDP_OK 0
 #define GDP_E_BADARG (-1)      /* null pointer, non-positive size, S / V / L above GDP_MAX_*, negative mem or other_mem, ... */
-#define GDP_E_UNSUPPORTED (-2) /* an input the device recurrence does not cover: mem <= 0 */
+#define GDP_E_UNSUPPORTED (-2) /* kept for callers built against earlier headers; no input is answered with it any more */
 #define GDP_E_NONFINITE (-3)   /* NaN or -inf in a cost array (the reference's result is then order-dependent) */
 #define GDP_E_NOMEM (-4)       /* device or host allocation failed */
 #define GDP_E_HIP (-5)         /* any other HIP runtime error; text in gdp_last_error() */
@@ -66,7 +66,10 @@ extern "C" {
  *   (the dictionary keys themselves are never used by the arithmetic).              */
 typedef struct gdp_problem {
     int32_t L, V, S;
-    const int32_t *mem;         /* [L][S]  memory cost in bins; every entry must be >= 1          */
+    const int32_t *mem;         /* [L][S]  memory cost in bins, >= 0.  An entry of 0 is computed with the reference's
+                                            in-place semantics (such a cell reads its own row, where lower strategies
+                                            already hold the layer's values: csrc/dp_core.cpp:58-73); a plan with such
+                                            entries runs one launch per layer                                   */
     const double *intra;        /* [L][S]                                                          */
     const double *inter;        /* [n_inter][S][S], row = source strategy, column = target        */
     const int32_t *inter_index; /* [L] layer -> matrix in `inter`; NULL means n_inter == L, identity */

@@ -53,6 +53,10 @@ def cases():
         c[f"rand_{i}"] = ("rand", {"seed": 2000 + i, "L": L, "S": S, "V": V})
         c[f"infeasible_{i}"] = ("infeasible", {"seed": 3000 + i, "L": L, "S": S, "V": V})
     c["galvatron_like"] = ("galvatron_like", {})
+    # memory costs of 0: the in-place update then reads its own, partly updated row (csrc/dp_core.cpp:58-73)
+    for i, (L, S, V, hi) in enumerate([(4, 6, 60, 2), (6, 22, 400, 3), (5, 44, 900, 1), (8, 64, 700, 4), (3, 65, 300, 2),
+                                       (7, 9, 513, 0), (10, 40, 2000, 6), (2, 88, 640, 1)]):
+        c[f"zeromem_{i}"] = ("zeromem", {"seed": 4000 + i, "L": L, "S": S, "V": V, "mem_hi": hi})
     return c
 
 
@@ -82,6 +86,15 @@ def build_case(builder: str, kw: dict) -> W.Instance:
         rng = np.random.Generator(np.random.PCG64(kw["seed"]))
         return W.random_instance(rng, kw["L"], kw["S"], kw["V"], mem_hi=max(1, kw["V"] // (kw["L"] + 1)),
                                  inf_frac=0.2, over_frac=0.15, n_keys=4)
+    if builder == "zeromem":
+        rng = np.random.Generator(np.random.PCG64(kw["seed"]))
+        # many zeros (mem in [0, mem_hi]), integer costs in the odd cases so that ties meet the in-row order
+        inst = W.random_instance(rng, kw["L"], kw["S"], kw["V"], mem_lo=0, mem_hi=kw["mem_hi"],
+                                 integer_costs=bool(kw["seed"] % 2), inf_frac=0.1 * (kw["seed"] % 3 == 0))
+        if kw["seed"] % 4 == 1:                          # some strategies with ordinary costs among the zeros
+            big = rng.uniform(size=inst.mem.shape) < 0.3
+            inst.mem[big] = rng.integers(1, max(2, kw["V"] // (kw["L"] + 1)), size=int(big.sum()))
+        return inst
     if builder == "galvatron_like":
         return galvatron_like()
     return getattr(W, builder)(**kw)

@@ -44,7 +44,8 @@ void make(Case &c, int L, int S, int V, int mem_hi, bool shared, unsigned flags)
     c.intra.resize((size_t)L * S);
     c.inter.resize((size_t)T * S * S);
     c.index.resize((size_t)L);
-    for (auto &m : c.mem) m = rnd_int(1, mem_hi);
+    const int mem_lo = rnd_int(0, 9) == 0 ? 0 : 1;    // now and then strategies with a memory cost of 0
+    for (auto &m : c.mem) m = rnd_int(mem_lo, mem_hi);
     for (auto &x : c.intra) x = rnd_unit() < 0.05 ? INFINITY : 1.0 + 19.0 * rnd_unit();
     for (auto &x : c.inter) x = 5.0 * rnd_unit();
     for (auto &x : c.index) x = rnd_int(0, T - 1);
@@ -132,7 +133,6 @@ int main()
         const gdp_problem *pp[1] = {&c.p};
         gdp_plan *plan = nullptr;
         auto create = [&]() { return gdp_plan_create(1, pp, &plan); };
-        c.mem[4] = 0;                  expect(create(), GDP_E_UNSUPPORTED, "mem == 0");
         c.mem[4] = -2;                 expect(create(), GDP_E_BADARG, "mem < 0");
         c.mem[4] = 3;
         c.other_mem[1] = -1;           expect(create(), GDP_E_BADARG, "other_mem < 0");

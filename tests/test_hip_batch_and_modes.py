@@ -351,9 +351,11 @@ def test_errors_surface_as_python_exceptions():
     intra = np.ones((L, S))
     inter = np.zeros((L, S, S))
     res = {1: np.full(L, -1, np.int32)}
-    bad = mem.copy(); bad[0, 0] = 0
-    with pytest.raises(_lib.UnsupportedInputError):
+    bad = mem.copy(); bad[0, 0] = -1
+    with pytest.raises(ValueError):
         shim.dynamic_programming_core(L, V, S, bad, None, None, inter, intra, {1: 0}, {1: 0.0}, res)
+    with pytest.raises(ValueError):                       # start row above the table
+        shim.dynamic_programming_core(L, V, S, mem, None, None, inter, intra, {1: -3}, {1: 0.0}, res)
     nan = intra.copy(); nan[1, 1] = np.nan
     with pytest.raises(ValueError):
         shim.dynamic_programming_core(L, V, S, mem, None, None, inter, nan, {1: 0}, {1: 0.0}, res)

@@ -67,6 +67,30 @@ def test_random_instances_against_oracle(n, shape, monkeypatch):
             monkeypatch.undo()
 
 
+ZERO_SHAPES = [(1, 1, 1), (3, 2, 9), (4, 7, 191), (5, 9, 193), (6, 11, 256), (3, 16, 383), (4, 22, 512), (3, 44, 1000),
+               (2, 64, 333), (2, 65, 200), (2, 88, 410), (2, 129, 131), (9, 5, 2048), (2, 257, 70), (1, 1024, 30)]
+
+
+@pytest.mark.parametrize("n,shape", list(enumerate(ZERO_SHAPES)))
+def test_memory_costs_of_zero_follow_the_in_place_order(n, shape):
+    """A strategy with mem == 0 reads its own row, where lower strategies already hold the layer's values
+    (csrc/dp_core.cpp:58-73; the oracle updates in place exactly like the reference).  All-zero layers,
+    zeros among ordinary costs, ties, +inf costs, single zero columns; whatever launch scheme is asked
+    for, costs-only and with the argmin table, full f and mark arrays compared."""
+    L, S, V = shape
+    for variant in range(4):
+        rng = np.random.Generator(np.random.PCG64([91, n, variant]))
+        hi = [0, 1, 3, max(1, V // (L + 1))][variant]
+        inst = W.random_instance(rng, L, S, V, mem_lo=0, mem_hi=hi, integer_costs=variant in (1, 3),
+                                 per_layer_inter=bool(variant % 2), inf_frac=0.15 if variant >= 2 else 0.0,
+                                 over_frac=0.1 if variant == 3 else 0.0, n_keys=min(4, 1 + variant))
+        if variant == 3:                                  # mostly ordinary costs, a sprinkling of zeros
+            inst.mem[(inst.mem == 0) & (rng.uniform(size=inst.mem.shape) < 0.7)] = max(1, V // (2 * L + 2))
+            inst.mem[rng.integers(0, L), rng.integers(0, S)] = 0
+        assert (inst.mem == 0).any()
+        _compare(inst, f"zero shape {shape} variant {variant}", launch=("fused", "per_layer", None, None)[variant])
+
+
 @pytest.mark.parametrize("shape", [(4, 8, 300), (3, 16, 200), (5, 11, 257), (3, 64, 150), (2, 44, 129)])
 def test_candidates_that_collide_only_after_the_intra_addition(shape, monkeypatch):
     """Transition costs that differ in the last bits under intra costs some 2^40 times larger: many

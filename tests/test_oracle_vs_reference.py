@@ -11,7 +11,8 @@ needs_ref = pytest.mark.skipif(not O.ref_available(), reason="oracle/_ref not bu
 
 CPU_GOLDEN = ([f"ties_{i}" for i in range(10)] + [f"rand_{i}" for i in range(10)] +
               [f"infeasible_{i}" for i in range(10)] + [f"cfg3_smallV_{i}" for i in range(8)] +
-              ["cfg2_small", "cfg4_small", "galvatron_like", "cfg0", "cfg0_other_time", "cfg1"])
+              ["cfg2_small", "cfg4_small", "galvatron_like", "cfg0", "cfg0_other_time", "cfg1"] +
+              [f"zeromem_{i}" for i in range(8)])
 
 
 @pytest.mark.parametrize("name", CPU_GOLDEN)
@@ -47,6 +48,7 @@ def test_oracle_vs_reference_build_random(seed):
     rng = np.random.Generator(np.random.PCG64(900 + seed))
     L, S, V = int(rng.integers(1, 9)), int(rng.integers(1, 70)), int(rng.integers(20, 900))
     inst = W.random_instance(rng, L, S, V, integer_costs=bool(seed % 2), mem_hi=max(1, V // (L + 1)),
+                             mem_lo=0 if seed % 5 == 0 else 1,     # memory costs of 0: the in-place update reads its own row
                              inf_frac=0.15 * (seed % 3 == 0), over_frac=0.1 * (seed % 4 == 0), n_keys=4)
     a = O.solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, keep=True)
     b = O.ref_solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, keep=True)

@@ -39,7 +39,7 @@ def test_static_entry_point_matches_gdp_solve_twice_in_a_row(golden):
         assert np.isfinite(want.total).any(), "the case should have feasible keys"
 
 
-@pytest.mark.parametrize("name", ["cfg0", "galvatron_like", "ties_3", "infeasible_2", "cfg4_small"])
+@pytest.mark.parametrize("name", ["cfg0", "galvatron_like", "ties_3", "infeasible_2", "cfg4_small", "zeromem_3", "zeromem_6"])
 def test_static_entry_point_on_golden_cases(golden, name):
     """... and against the reference's results for recorded cases, the Galvatron-like shape included."""
     rec = golden[name]
