@@ -15,18 +15,18 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
 * ``roofline``     for the relaxation kernel (the only kernel that matters): the fp64 vector
                    operations the kernel needs AND ISSUES for the relaxations it carries out -- one
                    addition and one minimum per relaxation plus one addition per cell, 2 + 1/S (intra
-                   is added after the minimum, which is exact because rounding is monotone); five per
-                   relaxation where the argmin table is stored, four + 1/S in the variant for small
-                   launches -- divided by the average launch duration measured with HIP events on the
+                   is added after the minimum, which is exact because rounding is monotone); four per
+                   relaxation where the argmin table is stored (two additions, compare, minimum; the
+                   select beside them is a 32-bit operation) -- divided by the average launch duration measured with HIP events on the
                    stream the kernel runs on; peak = 39.3 T operations/s = MI355X's published
                    78.6 TFLOP/s fp64 vector rate, which counts an FMA as two operations (additions and
                    minima cannot fuse) at the published 2.4 GHz.  ``frac`` is therefore a fraction of
                    the instruction-issue roof and cannot exceed 1.  ``frac_reference_ops`` counts the 3
                    operations per relaxation of the reference's loop body (two additions and one
                    comparison, csrc/dp_core.cpp:65-73) over the same time: it can exceed 1, because the
-                   kernel does not execute that work.  ``clock_ghz_under_load`` is the shader clock
-                   read from sysfs while the timed steps ran (null where the file is not readable;
-                   the SQ cycle counters in profiles/ give 2.05-2.10 GHz for cfg2).
+                   kernel does not execute that work.  ``clock_ghz_under_load`` is the shader clock the
+                   cycle counters in profiles/ give for this kernel under this workload (GRBM_GUI_ACTIVE
+                   over the dispatch duration; null where not profiled): the peak assumes 2.4 GHz.
                    ``traffic`` is the measured HBM-side byte count per launch from profiles/, given
                    only while the kernel sources still hash to what was profiled.
 * ``vs_baseline``  null: the reference publishes no number for this path.
@@ -95,48 +95,9 @@ def _traffic(key: str, tile: str):
     return nbytes, profile
 
 
-class _ClockSampler:
-    """Shader clock while the timed steps run: the level marked '*' in the amdgpu sysfs file
-    pp_dpm_sclk, sampled from a thread.  None where no such file is readable."""
-
-    def __init__(self):
-        import glob
-        self.paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
-        self.samples = []
-        self._stop = False
-        self._thread = None
-
-    def _read(self):
-        for p in self.paths:
-            try:
-                with open(p) as fh:
-                    for ln in fh:
-                        if "*" in ln:
-                            return float(ln.split(":")[1].strip().split("M")[0]) / 1e3
-            except (OSError, ValueError, IndexError):
-                continue
-        return None
-
-    def __enter__(self):
-        import threading
-        if self.paths:
-            def loop():
-                while not self._stop:
-                    v = self._read()
-                    if v:
-                        self.samples.append(v)
-                    time.sleep(0.002)
-            self._thread = threading.Thread(target=loop, daemon=True)
-            self._thread.start()
-        return self
-
-    def __exit__(self, *exc):
-        self._stop = True
-        if self._thread:
-            self._thread.join()
-
-    def ghz(self):
-        return sorted(self.samples)[len(self.samples) // 2] if self.samples else None
+# Shader clock under the relaxation kernel's load, from the cycle counters in profiles/ (GRBM_GUI_ACTIVE
+# over the dispatch duration): the published peak assumes 2.4 GHz.
+PROFILED_CLOCK_GHZ = {"cfg2": 2.08, "cfg3": 2.17}
 
 
 def _bit_exact(workload: str, probs) -> bool | None:
@@ -245,6 +206,9 @@ def main() -> int:
     ap.add_argument("--row-skipping", action="store_true",
                     help="time the library's default (rows that need no arithmetic are filled or left out) instead "
                          "of carrying out every relaxation; the line says so and gives the executed fraction")
+    ap.add_argument("--mark-table", action="store_true",
+                    help="time the mode that stores the reference's argmin table while relaxing (GDP_KEEP_MARKS) as the "
+                         "headline leg (profiling runs of that mode); the line says so")
     ap.add_argument("--headline-only", action="store_true",
                     help="leave out the row-skipping and mark-table legs (profiling runs: the trace then holds the "
                          "headline's launches alone)")
@@ -288,12 +252,11 @@ def main() -> int:
             for _ in range(warmup):
                 plan.run(0)
             device_sync()
-            with _ClockSampler() as clock:
-                t0 = time.perf_counter()
-                for _ in range(steps):
-                    plan.run(0)                       # synchronises the plan's stream before returning
-                device_sync()
-                wall = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                plan.run(0)                       # synchronises the plan's stream before returning
+            device_sync()
+            wall = time.perf_counter() - t0
             tm = plan.run(2)                       # per-launch HIP events on the plan's stream
             t1 = plan.run(1)
             plan.fetch()
@@ -317,9 +280,10 @@ def main() -> int:
         launches = tm.relax_launches
         avg_launch_s = tm.relax_ms * 1e-3 / launches
         # fp64 vector operations the kernel issues per relaxation: v_add_f64 + v_min_f64, plus one addition
-        # per cell (1/S); with the argmin table two additions, compare, select, minimum; the variant for
-        # small per-layer launches spends two more (v_readlane) on spreading the transition costs
-        issued = 5.0 if keep_marks else (4.0 if tm.latency_variant else 2.0) + 1.0 / insts[0].S
+        # per cell (1/S); with the argmin table two additions, a compare and a minimum (its select is a
+        # 32-bit operation, like the two v_readlane per relaxation of the variant for small per-layer
+        # launches: not fp64 work, not counted)
+        issued = 4.0 if keep_marks else 2.0 + 1.0 / insts[0].S
         per_launch_s = tm.executed / launches / avg_launch_s
         return {
             "insts": insts, "probs": probs, "relaxations": relax, "ms_per_step": wall / steps * 1e3,
@@ -334,7 +298,8 @@ def main() -> int:
             "tile_key": "%dx%d" % (tm.tile_ts, tm.tile_r),
             "kernel": "gdp_relax_fused_kernel" if tm.fused else
                       ("gdp_relax_kernel (latency variant)" if tm.latency_variant else "gdp_relax_kernel"),
-            "clock_ghz": clock.ghz(), "bit_exact": bit_exact,
+            "clock_ghz": PROFILED_CLOCK_GHZ.get(workload) if compute_all and not keep_marks else None,
+            "bit_exact": bit_exact,
         }
 
     def fractions(mm):
@@ -342,11 +307,12 @@ def main() -> int:
                 "frac_reference_ops": mm["tops_reference"] / PEAK_FP64_VALU_TFLOPS,
                 "frac_hbm": mm["gbs"] / PEAK_HBM_GBS}
 
-    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping, host_leg=not a.headline_only,
-                check=True)
+    m = measure(a.workload, a.steps, a.warmup, compute_all=not a.row_skipping, keep_marks=a.mark_table,
+                host_leg=not a.headline_only, check=True)
     insts = m["insts"]
     first = insts[0]
-    traffic, traffic_source = _traffic(a.workload + ("+row_skipping" if a.row_skipping else ""), m["tile_key"])
+    traffic, traffic_source = _traffic(a.workload + ("+row_skipping" if a.row_skipping else "") +
+                                       ("+mark_table" if a.mark_table else ""), m["tile_key"])
     fr = fractions(m)
     line = {
         "metric": "min-plus relaxations/s (L*V*S^2)", "value": m["value"], "unit": "relaxations/s",
@@ -354,7 +320,9 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": a.workload, "instances": len(insts), "L": first.L if len(insts) == 1 else "32/pp",
                    "S": first.S, "V": first.V, "relaxations_per_step": m["relaxations"],
-                   "argmin": "recomputed on the backtrack (costs-only relaxation)", "search_wall_ms_device": m["device_ms"],
+                   "argmin": ("stored while relaxing (one byte per cell)" if a.mark_table else
+                              "recomputed on the backtrack (costs-only relaxation)"),
+                   "search_wall_ms_device": m["device_ms"],
                    "search_wall_ms_from_host_arrays": m["host_ms"], "launch_scheme": m["scheme"],
                    "register_tile": m["tile"],
                    "relaxations_executed_fraction": m["executed_fraction"], "bit_exact": m["bit_exact"],

@@ -769,44 +769,34 @@ __global__ __launch_bounds__(256) void gdp_zero_pass_kernel(const GdpDevInst *in
 }
 
 // ---- wavefront (value, index) reduction: lower value wins, equal values -> lower index ----------
-__device__ __forceinline__ double swz_f64(double x, int pattern_sel)
+// One combining step through the data-parallel-primitive path of the vector ALU (no LDS round trip):
+// every enabled lane looks at the pair of the lane that CTRL names and keeps the better of the two;
+// lanes that CTRL gives no source, and rows outside ROW_MASK, see their own pair again and keep it.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void argmin_step(double &val, int &idx)
 {
-    int lo = __double2loint(x), hi = __double2hiint(x);
-    switch (pattern_sel) {  // ds_swizzle bit-mode: and=0x1f, or=0, xor=1<<k, within groups of 32 lanes
-        case 0: lo = __builtin_amdgcn_ds_swizzle(lo, 0x041f); hi = __builtin_amdgcn_ds_swizzle(hi, 0x041f); break;
-        case 1: lo = __builtin_amdgcn_ds_swizzle(lo, 0x081f); hi = __builtin_amdgcn_ds_swizzle(hi, 0x081f); break;
-        case 2: lo = __builtin_amdgcn_ds_swizzle(lo, 0x101f); hi = __builtin_amdgcn_ds_swizzle(hi, 0x101f); break;
-        case 3: lo = __builtin_amdgcn_ds_swizzle(lo, 0x201f); hi = __builtin_amdgcn_ds_swizzle(hi, 0x201f); break;
-        default: lo = __builtin_amdgcn_ds_swizzle(lo, 0x401f); hi = __builtin_amdgcn_ds_swizzle(hi, 0x401f); break;
-    }
-    return __hiloint2double(hi, lo);
-}
-__device__ __forceinline__ int swz_i32(int x, int pattern_sel)
-{
-    switch (pattern_sel) {
-        case 0: return __builtin_amdgcn_ds_swizzle(x, 0x041f);
-        case 1: return __builtin_amdgcn_ds_swizzle(x, 0x081f);
-        case 2: return __builtin_amdgcn_ds_swizzle(x, 0x101f);
-        case 3: return __builtin_amdgcn_ds_swizzle(x, 0x201f);
-        default: return __builtin_amdgcn_ds_swizzle(x, 0x401f);
-    }
-}
-
-__device__ __forceinline__ void wave_argmin(double &val, int &idx)
-{
-#pragma unroll
-    for (int k = 0; k < 5; ++k) {
-        const double ov = swz_f64(val, k);
-        const int oi = swz_i32(idx, k);
-        if (ov < val || (ov == val && oi < idx)) { val = ov; idx = oi; }
-    }
-    // halves of the wavefront: lanes l and l^32 (ds_swizzle works within 32 lanes)
-    const int partner = (int)((threadIdx.x & 63u) ^ 32u) << 2;
-    const int olo = __builtin_amdgcn_ds_bpermute(partner, __double2loint(val));
-    const int ohi = __builtin_amdgcn_ds_bpermute(partner, __double2hiint(val));
-    const int oi = __builtin_amdgcn_ds_bpermute(partner, idx);
+    const int lo = __double2loint(val), hi = __double2hiint(val);
+    const int olo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+    const int ohi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+    const int oi = __builtin_amdgcn_update_dpp(idx, idx, CTRL, ROW_MASK, 0xf, false);
     const double ov = __hiloint2double(ohi, olo);
     if (ov < val || (ov == val && oi < idx)) { val = ov; idx = oi; }
+}
+
+// On return every lane holds the wavefront's best pair.  Within each row of 16 lanes the pairs are
+// folded towards lane 15 (shifts by 1, 2, 4, 8), lane 15 of rows 0 and 2 is then broadcast into rows 1
+// and 3, lane 31 into rows 2 and 3; lane 63 ends up with the result, which is read out of it.
+__device__ __forceinline__ void wave_argmin(double &val, int &idx)
+{
+    argmin_step<0x111, 0xf>(val, idx);   // row_shr:1
+    argmin_step<0x112, 0xf>(val, idx);   // row_shr:2
+    argmin_step<0x114, 0xf>(val, idx);   // row_shr:4
+    argmin_step<0x118, 0xf>(val, idx);   // row_shr:8
+    argmin_step<0x142, 0xa>(val, idx);   // row_bcast:15 into rows 1 and 3
+    argmin_step<0x143, 0xc>(val, idx);   // row_bcast:31 into rows 2 and 3
+    idx = __builtin_amdgcn_readlane(idx, 63);
+    val = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(val), 63),
+                           __builtin_amdgcn_readlane(__double2loint(val), 63));
 }
 
 // Epilogue of csrc/dp_core.cpp:78-117 for one key per wavefront: first argmin of the start row,
