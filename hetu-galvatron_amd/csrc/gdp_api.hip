@@ -676,10 +676,18 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->num_cu = pl->dry_num_cu;
         pl->lds_per_cu = pl->dry_lds_per_cu;
     } else {
-        hipDeviceProp_t prop;
-        GDP_HIP(hipGetDeviceProperties(&prop, pl->device));
-        pl->num_cu = prop.multiProcessorCount;
-        pl->lds_per_cu = prop.maxSharedMemoryPerMultiProcessor;
+        // asked once per device: the call costs as much as laying out a small plan
+        static std::mutex mu;
+        static std::vector<std::pair<int, size_t>> known;   // per device: {CUs, LDS bytes per CU}, {0, 0} = not asked yet
+        std::lock_guard<std::mutex> lk(mu);
+        if ((size_t)pl->device >= known.size()) known.resize((size_t)pl->device + 1, {0, 0});
+        if (known[(size_t)pl->device].first == 0) {
+            hipDeviceProp_t prop;
+            GDP_HIP(hipGetDeviceProperties(&prop, pl->device));
+            known[(size_t)pl->device] = {prop.multiProcessorCount, (size_t)prop.maxSharedMemoryPerMultiProcessor};
+        }
+        pl->num_cu = known[(size_t)pl->device].first;
+        pl->lds_per_cu = known[(size_t)pl->device].second;
     }
     std::vector<HostInst> inst((size_t)n);
     for (int i = 0; i < n; ++i) {

@@ -97,10 +97,11 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
 // 0.2 us when it misses the scalar cache -- nothing when other waves fill the gap, the whole run time
 // of a layer when there are one or two waves per SIMD.  Here nothing inside a trip waits for a
 // scalar load:
-//   - the row of transition costs travels as a vector load (lane j holds column j), NS steps ahead
-//     like the cost rows -- vector loads return in order, so a wait can leave the younger ones in
-//     flight -- and is spread to scalar registers with v_readlane (2*TS more vector instructions per
-//     step; instruction issue is not what such a launch is short of);
+//   - the row of transition costs travels as a vector load (lane j of every row of 16 lanes holds
+//     column j), NS steps ahead like the cost rows -- vector loads return in order, so a wait can
+//     leave the younger ones in flight -- and is spread over the lanes with one 64-bit DPP move per
+//     column (v_mov_b64 row_newbcast: lane j of a row to the whole row; TS more vector instructions
+//     per step -- instruction issue is not what such a launch is short of);
 //   - the row offsets of a whole trip are fetched with the previous trip's.
 // Same arithmetic in the same order as relax_task, hence the same bits.
 //
@@ -124,7 +125,8 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
     const double *it = uload(&Y->it) + s0 + (int64_t)part * SU * SP;
     const int64_t u0 = (int64_t)tile * (64 * R);
     const unsigned lane_bytes = lane * 8u;
-    const unsigned col_bytes = (lane < (unsigned)TS ? lane : (unsigned)(TS - 1)) * 8u;
+    static_assert(TS <= 16, "a row of 16 lanes holds the transition costs of a step");
+    const unsigned col_bytes = ((lane & 15u) < (unsigned)TS ? (lane & 15u) : (unsigned)(TS - 1)) * 8u;
 
     double best[R][TS];
     int arg_unused[1][1];
@@ -174,12 +176,9 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
             double sc[TS];
-            {
-                const int lo = __double2loint(scv[u]), hi = __double2hiint(scv[u]);
 #pragma unroll
-                for (int j = 0; j < TS; ++j)
-                    sc[j] = __hiloint2double(__builtin_amdgcn_readlane(hi, j), __builtin_amdgcn_readlane(lo, j));
-            }
+            for (int j = 0; j < TS; ++j)   // lane j of every row of 16 lanes holds column j: one move spreads it
+                asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(sc[j]) : "v"(scv[u]), "n"(j));
             relax_cols<TS, R, false, 0, TS>(best, arg_unused, fp[u], sc, add_unused, sp + u);
             GDP_SCHED_FENCE();
             {
