@@ -201,8 +201,8 @@ def _cpu_baseline_all_cores(budget_s: float = 8.0):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--row-skipping", action="store_true",
@@ -351,7 +351,8 @@ def main() -> int:
                    "roofline_frac_valu_fp64": ff["frac"], "issued_ops_per_relaxation": mm["issued_per_relaxation"],
                    "roofline_frac_valu_fp64_reference_ops": ff["frac_reference_ops"],
                    "roofline_frac_hbm": ff["frac_hbm"], "avg_launch_ms": mm["avg_launch_ms"],
-                   "launches_per_step": mm["launches"], "bit_exact": mm["bit_exact"]}
+                   "launches_per_step": mm["launches"], "traffic": _traffic(w, mm["tile_key"])[0],
+                   "bit_exact": mm["bit_exact"]}
     if also:
         line["also"] = also
     if a.row_skipping:

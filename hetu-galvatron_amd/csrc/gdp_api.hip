@@ -1067,6 +1067,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 y.src = d.H + (int64_t)(l % h.nbuf) * d.hstride;
                 y.dst = d.H + (int64_t)((l + 1) % h.nbuf) * d.hstride + h.P;
                 y.ro = d.roff + (int64_t)l * rows;
+                memcpy(y.ro_head, reinterpret_cast<const int64_t *>(stage.data() + h.off_roff) + (size_t)l * rows,
+                       sizeof(y.ro_head));
                 y.it = d.inter + (int64_t)mat * rows * h.SP;
                 y.ia = d.intra + (int64_t)l * h.SP;
                 y.m = d.M ? d.M + (int64_t)l * h.S * h.ldm : nullptr;

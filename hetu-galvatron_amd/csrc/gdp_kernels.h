@@ -27,7 +27,7 @@
 //   mem    L rows of S int32, as given.
 //
 // The relaxation kernels do not read the instance record at all: everything one (instance, layer)
-// step needs is precomputed into one 128-byte GdpDevLayer record (one scalar load away from the
+// step needs is precomputed into one 256-byte GdpDevLayer record (one scalar load away from the
 // kernel arguments), in a table of n_inst x max_L records per group of instances.
 //   dep    ceil(max mem[l] / tile rows): a reader of layer l's output at tile t touches tiles
 //          [t-dep, t].
@@ -78,8 +78,9 @@ struct GdpDevLayer {
     int32_t S, SU, SP, ntile;
     int32_t dep, lo, hi;  // see above; an entry of an instance without this layer has lo = 0, hi = -1
     int32_t pad_[9];
+    int64_t ro_head[16];  // copy of ro[0..16): a task that starts from them needs no second round trip
 };
-static_assert(sizeof(GdpDevLayer) == 128, "one record = two 64-byte scalar loads");
+static_assert(sizeof(GdpDevLayer) == 256, "one record = four 64-byte scalar loads");
 
 // Bookkeeping of one fused (all layers) launch over a group of instances.  Passed to the kernel by
 // value: its fields arrive with the kernel arguments, one dependent load fewer at the start of every

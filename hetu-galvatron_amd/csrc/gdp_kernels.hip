@@ -110,19 +110,47 @@ __device__ __forceinline__ void relax_cols(double (&best)[R][TS], int (&arg)[ARG
 // dependent steps K times where there are wave slots to spare.  The partial minima meet in LDS; the
 // minimum of the parts is the minimum over all sources exactly (min is associative and commutative),
 // and the wave of part j % K adds intra to column j and stores it.
+// What a task of the latency variant needs from its layer record, fetched by the caller in one round
+// of scalar loads (with the band the caller itself needs) and kept in scalar registers.
+struct LatHead {
+    const double *src, *it, *ia;
+    double *dst;
+    const int64_t *ro;
+    int64_t ld;
+    int S, SU, SP, lo, hi;
+    int64_t head[2 * 8];   // ro[0..16)
+};
+
+__device__ __forceinline__ LatHead load_lat_head(const GdpDevLayer *Y)
+{
+    LatHead h;
+    h.src = uload(&Y->src); h.dst = uload(&Y->dst); h.ro = uload(&Y->ro); h.it = uload(&Y->it);
+    h.ia = uload(&Y->ia); h.ld = uload(&Y->ld);
+    h.S = uload(&Y->S); h.SU = uload(&Y->SU); h.SP = uload(&Y->SP); h.lo = uload(&Y->lo); h.hi = uload(&Y->hi);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) h.head[u] = uload(&Y->ro_head[u]);
+    // all of it has arrived before the first branch: left alone, the compiler fetches the fields where
+    // they are first used, one dependent round trip after the other
+#pragma unroll
+    for (int u = 0; u < 16; ++u) asm volatile("" : "+s"(h.head[u]));
+    asm volatile("" : "+s"(h.src), "+s"(h.dst), "+s"(h.ro), "+s"(h.it), "+s"(h.ia), "+s"(h.ld));
+    asm volatile("" : "+s"(h.S), "+s"(h.SU), "+s"(h.SP), "+s"(h.lo), "+s"(h.hi));
+    return h;
+}
+
 template <int TS, int R, bool PUBLISH, int K>
-__device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned tile, unsigned vtb, unsigned lane)
+__device__ __forceinline__ void relax_task_lat(const LatHead &H, unsigned tile, unsigned vtb, unsigned lane)
 {
     constexpr int NS = 8;
     static_assert(GDP_SRC_UNROLL_LAT % NS == 0 && GDP_SRC_PAD >= 2 * NS, "padding of roff / inter");
     static_assert(K == 1 || (R == 1 && GDP_WAVES_PER_BLOCK % K == 0), "parts of one task share a workgroup");
     const unsigned tb = vtb / K, part = vtb % K;
-    const int SU = uload(&Y->SU) / K;   // a multiple of NS in the groups this variant runs for
-    const int SP = uload(&Y->SP);
-    const double *src = uload(&Y->src);
-    const int64_t *ro = uload(&Y->ro) + part * SU;
+    const int SU = H.SU / K;   // a multiple of NS in the groups this variant runs for
+    const int SP = H.SP;
+    const double *src = H.src;
+    const int64_t *ro = H.ro + part * SU;
     const int s0 = tb * TS;
-    const double *it = uload(&Y->it) + s0 + (int64_t)part * SU * SP;
+    const double *it = H.it + s0 + (int64_t)part * SU * SP;
     const int64_t u0 = (int64_t)tile * (64 * R);
     const unsigned lane_bytes = lane * 8u;
     static_assert(TS <= 16, "a row of 16 lanes holds the transition costs of a step");
@@ -138,15 +166,22 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
 #pragma unroll
     for (int j = 0; j < TS; ++j) add_unused[j] = 0.0;
 
-    double fp[NS][R], scv[NS];
+    double fp[NS][R], scv[NS], iav;
     int64_t ocur[NS], onext[NS];
     const double *itp = it;   // row of the transition matrix that the next request fetches
     {
         int64_t o0[NS];
+        if constexpr (K == 1) {
 #pragma unroll
-        for (int u = 0; u < NS; ++u) o0[u] = uload(ro + u);
+            for (int u = 0; u < NS; ++u) o0[u] = H.head[u];
 #pragma unroll
-        for (int u = 0; u < NS; ++u) ocur[u] = uload(ro + NS + u);
+            for (int u = 0; u < NS; ++u) ocur[u] = H.head[NS + u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < NS; ++u) o0[u] = uload(ro + u);
+#pragma unroll
+            for (int u = 0; u < NS; ++u) ocur[u] = uload(ro + NS + u);
+        }
         GDP_SCHED_FENCE();
         unsigned lb = lane_bytes, cb = col_bytes;
         GDP_PIN_LANE(lb);
@@ -163,6 +198,12 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
             itp += SP;
             GDP_SCHED_FENCE();
         }
+        // the intra costs of the target columns travel like a row of transition costs (lane j of
+        // every row of 16 lanes holds column j) and are long there when the loop ends
+        const double *qa = H.ia + s0;
+        asm volatile("" : "+s"(qa));
+        iav = lane_load(qa, cb, 0);
+        GDP_SCHED_FENCE();
     }
     const int64_t *rop = ro + 2 * NS;
     for (int sp = 0; sp < SU; sp += NS) {
@@ -170,8 +211,14 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
         GDP_PIN_LANE(lb);
         GDP_PIN_LANE(cb);
         // row offsets for the requests of the next trip: a whole trip ahead of their use
+        {
+            typedef long long trip_t __attribute__((ext_vector_type(NS)));   // one wide scalar load
+            typedef trip_t trip_a8 __attribute__((aligned(8)));
+            const trip_t t =
+                *reinterpret_cast<const __attribute__((address_space(4))) trip_a8 *>(reinterpret_cast<uintptr_t>(rop));
 #pragma unroll
-        for (int u = 0; u < NS; ++u) onext[u] = uload(rop + u);
+            for (int u = 0; u < NS; ++u) onext[u] = t[u];
+        }
         GDP_SCHED_FENCE();
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
@@ -217,20 +264,16 @@ __device__ __forceinline__ void relax_task_lat(const GdpDevLayer *Y, unsigned ti
             }
         }
     }
-    const GdpDevLayer *Z = Y;
-    asm volatile("" : "+s"(Z));
-    {
-        const double *iz = uload(&Z->ia) + s0;
 #pragma unroll
-        for (int j = 0; j < TS; ++j) {
-            const double a = uload(iz + j);
+    for (int j = 0; j < TS; ++j) {
+        double a;
+        asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(a) : "v"(iav), "n"(j));
 #pragma unroll
-            for (int r = 0; r < R; ++r) best[r][j] += a;
-        }
+        for (int r = 0; r < R; ++r) best[r][j] += a;
     }
-    const int64_t ld = uload(&Z->ld);
-    const int nvalid = uload(&Z->S) - s0;
-    double *drow = uload(&Z->dst) + (int64_t)s0 * ld + u0;
+    const int64_t ld = H.ld;
+    const int nvalid = H.S - s0;
+    double *drow = H.dst + (int64_t)s0 * ld + u0;
 #pragma unroll
     for (int j = 0; j < TS; ++j) {
         if (j < nvalid) {
@@ -461,23 +504,31 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     // out, every XCD getting one contiguous range of them (equal work per XCD, neighbouring budget
     // rows in one L2); the blocks after those fill the tiles below lo; tiles above hi are left alone.
     // (A table entry of an instance that has no such layer has hi = -1 and lo = 0.)
-    const int lo = uload(&Y->lo), hi = uload(&Y->hi);
-    const unsigned live_tasks = hi >= lo ? (unsigned)(hi - lo + 1) * ntb : 0u;
-    const unsigned live_blocks = ((live_tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK + 7u) & ~7u;
-    if (blockIdx.x < live_blocks) {
+    if constexpr (LAT > 0) {
+        const LatHead H = load_lat_head(Y);
+        const unsigned live_tasks = H.hi >= H.lo ? (unsigned)(H.hi - H.lo + 1) * ntb : 0u;
+        const unsigned live_blocks = ((live_tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK + 7u) & ~7u;
+        if (blockIdx.x >= live_blocks) return;   // (costs only: the rows below the band were filled when the plan was made)
         const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
         if (task >= live_tasks) return;
         const unsigned t = task / ntb;
-        if constexpr (LAT > 0)
-            relax_task_lat<TS, R, false, LAT>(Y, (unsigned)lo + t, task - t * ntb, lane);
-        else
+        relax_task_lat<TS, R, false, LAT>(H, (unsigned)H.lo + t, task - t * ntb, lane);
+    } else {
+        const int lo = uload(&Y->lo), hi = uload(&Y->hi);
+        const unsigned live_tasks = hi >= lo ? (unsigned)(hi - lo + 1) * ntb : 0u;
+        const unsigned live_blocks = ((live_tasks + GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK + 7u) & ~7u;
+        if (blockIdx.x < live_blocks) {
+            const unsigned task = xcd_swizzle(blockIdx.x, live_blocks) * GDP_WAVES_PER_BLOCK + wave;
+            if (task >= live_tasks) return;
+            const unsigned t = task / ntb;
             relax_task<TS, R, false, ARG>(Y, (unsigned)lo + t, task - t * ntb, lane);
-    } else if constexpr (ARG) {  // (costs only: those rows were filled when the plan was made)
-        const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
-        const unsigned t = task / ntb;
-        const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
-        if ((int)t > top) return;
-        fill_task<TS, R, false, ARG>(Y, t, task - t * ntb, lane);
+        } else if constexpr (ARG) {  // (costs only: those rows were filled when the plan was made)
+            const unsigned task = (blockIdx.x - live_blocks) * GDP_WAVES_PER_BLOCK + wave;
+            const unsigned t = task / ntb;
+            const int top = lo - 1 < hi ? lo - 1 : hi;  // fill tiles 0 .. min(lo-1, hi)
+            if ((int)t > top) return;
+            fill_task<TS, R, false, ARG>(Y, t, task - t * ntb, lane);
+        }
     }
 }
 

@@ -183,6 +183,7 @@ void build(const gdp_problem *p, const Layout &y, unsigned char *base)
         r.src = d.H + (int64_t)(l % 2) * d.hstride;
         r.dst = d.H + (int64_t)((l + 1) % 2) * d.hstride + y.P;
         r.ro = d.roff + (int64_t)l * y.rows;
+        memcpy(r.ro_head, ro + (size_t)l * y.rows, sizeof(r.ro_head));
         r.it = d.inter + (int64_t)mat * y.rows * y.SP;
         r.ia = d.intra + (int64_t)l * y.SP;
         r.m = d.M + (int64_t)l * y.S * y.ldm;
