@@ -183,6 +183,7 @@ struct Lane {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    hipEvent_t ev_back = nullptr;  // after the copy of the results (a flow run queues more work behind it)
     char *back = nullptr;  // page-locked host memory the results are copied into
     size_t back_bytes = 0;
     char *up = nullptr;    // page-locked host memory the inputs' device layout is built in (may be absent)
@@ -196,6 +197,7 @@ void lane_release(Lane &ln)  // the lane's device is current
 {
     if (ln.ev_begin) (void)hipEventDestroy(ln.ev_begin);
     if (ln.ev_end) (void)hipEventDestroy(ln.ev_end);
+    if (ln.ev_back) (void)hipEventDestroy(ln.ev_back);
     if (ln.stream) (void)hipStreamDestroy(ln.stream);
     if (ln.back) (void)hipHostFree(ln.back);
     if (ln.up) (void)hipHostFree(ln.up);
@@ -238,6 +240,7 @@ hipError_t lane_take(int device, size_t back_bytes, size_t up_bytes, Lane *out)
         e = hipStreamCreateWithFlags(&ln.stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_begin);
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_end);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&ln.ev_back, hipEventDisableTiming);
     }
     if (e == hipSuccess) e = pinned_reserve(&ln.back, &ln.back_bytes, back_bytes, 65536);
     if (e == hipSuccess && up_bytes <= UPLOAD_PINNED_MAX) e = pinned_reserve(&ln.up, &ln.up_bytes, up_bytes, (size_t)1 << 20);
@@ -336,6 +339,10 @@ struct Group {  // instances with the same S, sorted by L descending
     int max_V = 0;
     int latency = 0;                // per-layer launches use the variant for launches with few waves: 0, or the
                                     // number of waves (1, 2, 4) that share the source strategies of a task
+    int flow_nsrc = 0;              // flow launch: source strategies per wave (SU = flow_nsrc * latency)
+    bool lat_ok = true;             // SU suits the latency variant of the per-layer kernel (a multiple of 8 * latency)
+    unsigned flow_lds = 0;          // flow launch: dynamic LDS that holds the workgroups per CU down (never touched)
+    int flow_blocks = 0;            // flow launch: workgroups of the widest band (wave tasks incl. the parts of split ones)
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
     std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
     size_t off_rows = 0;
@@ -430,8 +437,15 @@ struct gdp_plan {
     double executed = 0;     // relaxations actually carried out (tiles inside the bands)
     bool skip = true;        // GDP_OPT_SKIP: use the bands (off: every tile of every layer is computed)
     bool ran = false;
+    bool flow_clean = false;      // every cell a flow launch writes holds NaN and the abort flag zero (nothing has run since)
+    bool one_shot = false;        // the plan runs once (gdp_solve_batch): nothing is prepared for a next run
+    bool wait_back = false;       // the last run queued work behind its results: run_finish waits for lane.ev_back only
     bool holds_fused = false;     // between run_enqueue and run_finish of a fused run: this plan has the turn
     bool fused = true;            // one launch for all layers instead of one per layer
+    bool flow = false;            // one launch for all layers whose tasks wait on the cost cells themselves (small
+                                  // plans; see gdp_relax_flow_kernel); only with fused off
+    bool flow_ready = false;      // the plan was laid out for it: closed bands, latency tile, NaN in the bands
+    int flow_override = -1;       // GALVATRON_DP_FLOW=0|1: never / wherever the layout allows
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
     int64_t spin_limit = 1 << 18; // polls a waiting wave makes before the launch is abandoned: about a second
@@ -570,7 +584,12 @@ void destroy(gdp_plan *pl)
 //      u + sum_{k>=l} mem[k][s_k] = v0 for some choice, hence u <= max v0 - sum_{k>=l} min_s mem[k][s];
 //      rows above are never read by a row inside the band of the next layer, nor by the epilogue.
 // `skip` off (or exports requested, for hi) gives the full range.
-void fill_bands(const gdp_problem *q, const HostInst &h, int tile_rows, bool skip, int32_t *dep, double *executed)
+// closed: hi is raised, where needed, to the tile that holds the highest row read by the band of the
+//      next layer.  (A tile is computed whole, so the band of layer l+1 reads up to tile_rows - 1 rows
+//      beyond what any path needs; those cells matter to no result, but a flow launch waits for every
+//      cell it reads and must find each of them written.)
+void fill_bands(const gdp_problem *q, const HostInst &h, int tile_rows, bool skip, int32_t *dep, double *executed,
+                bool closed = false)
 {
     std::vector<int64_t> minfin((size_t)h.L), minany((size_t)h.L);
     for (int l = 0; l < h.L; ++l) {
@@ -594,6 +613,12 @@ void fill_bands(const gdp_problem *q, const HostInst &h, int tile_rows, bool ski
     std::vector<int64_t> ub((size_t)h.L + 1);
     ub[(size_t)h.L] = v0max;
     for (int l = h.L - 1; l >= 0; --l) ub[(size_t)l] = ub[(size_t)l + 1] - minany[(size_t)l];
+    if (closed && !full)   // layer l+1 reads row u - mem[l][s'] of layer l's output for every row u of its own band
+        for (int l = h.L - 2; l >= 0; --l) {
+            if (ub[(size_t)l + 1] < 0) continue;
+            const int64_t top = std::min<int64_t>(h.ntile - 1, ub[(size_t)l + 1] / tile_rows) * tile_rows + tile_rows - 1;
+            ub[(size_t)l] = std::max(ub[(size_t)l], top - minany[(size_t)l]);
+        }
     for (int l = 0; l < h.L; ++l) {
         int64_t lo = skip ? std::min<int64_t>(reach, h.V) / tile_rows : 0;
         int64_t hi = h.ntile - 1;
@@ -643,6 +668,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     if (const char *e = getenv("GALVATRON_DP_TILE_R")) pl->tile_r_override = atoi(e);
     if (const char *e = getenv("GALVATRON_DP_LATENCY_VARIANT")) pl->latency_override = std::max(0, atoi(e));
     if (const char *e = getenv("GALVATRON_DP_CHUNK")) pl->chunk_override = atoi(e);
+    if (const char *e = getenv("GALVATRON_DP_FLOW")) pl->flow_override = atoi(e) != 0;
     if (const char *e = getenv("GALVATRON_DP_OCCUPANCY_CAP")) {
         pl->no_occupancy_cap = atoi(e) == 0;
         pl->occupancy_cap_override = atoi(e);
@@ -804,7 +830,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->groups.push_back(g);
         i = j;
     }
-    if (!fused_preset) {
+    double band_frac = 1.0;   // share of the relaxations that lie inside the bands
+    if (!fused_preset || pl->flow_override != 0) {
         // One launch for all layers pays off once a layer holds about two block tasks that carry
         // arithmetic per CU (measured: 950 per layer, 0.48 ms against 0.58 ms; 128 per layer, 0.23 ms
         // against 0.17 ms): the launch gaps and the ramp up and down of every layer go away, and layers
@@ -821,16 +848,27 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 all += (double)h.L * h.V * (double)h.S * h.S;
             }
         }
-        pl->fused = first_layer * (all > 0 ? live / all : 1.0) >= 2.0 * pl->num_cu;
+        band_frac = all > 0 ? live / all : 1.0;
+        if (!fused_preset) pl->fused = first_layer * band_frac >= 2.0 * pl->num_cu;
     }
     // Launches that small run one or two waves per SIMD, and what they wait for is memory latency, not
     // instruction issue: their narrowest tile has a variant built for that (measured, 16 layers, one
     // instance: S=22 V=16384 0.176 -> 0.126 ms, S=44 V=16384 0.241 -> 0.208, S=64 V=4096 0.284 -> 0.192;
     // with all layers in one launch, or on larger problems, it is the slower one).
+    // Plans that small run all their layers in one launch that waits on the cost cells themselves
+    // (gdp_relax_flow_kernel) -- unless the caller asked for a launch scheme: per-layer launches are also
+    // what a shared device wants, since they never wait.  GALVATRON_DP_FLOW=1 asks for it wherever the
+    // layout allows (costs only, no memory cost of 0, the tile of the latency variant).
+    bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused) : !fused_preset;
+    want_flow = want_flow && !pl->fused && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65535;
+    for (const Group &g : pl->groups)
+        want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
+    pl->flow = pl->flow_ready = want_flow;
     for (Group &g : pl->groups) {
         const GdpVariant &v = GDP_VARIANTS[g.variant];
         bool on = !pl->fused && !pl->keep_marks && v.ts == GDP_LAT_TS && v.r == GDP_LAT_R;
         if (pl->latency_override >= 0) on = g.latency_possible(pl->keep_marks) && pl->latency_override != 0;
+        if (pl->flow_ready) on = true;
         g.latency = 0;
         if (on) {
             // With many sources and wave slots to spare, the sources of a task are split over 2 or 4 waves:
@@ -844,8 +882,39 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             const int64_t room = (int64_t)pl->num_cu * 4 * 3;  // three waves per SIMD
             g.latency = g.S < 32 ? 1 : tasks * 4 <= room ? 4 : tasks * 2 <= room ? 2 : 1;
             if (pl->latency_override >= 1) g.latency = pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1;
-            for (int k = g.first; k < g.first + g.count; ++k)
-                inst[(size_t)k].SU = (int)align_up((size_t)inst[(size_t)k].S, (size_t)GDP_SRC_UNROLL_LAT * g.latency);
+            int su = (int)align_up((size_t)g.S, (size_t)GDP_SRC_UNROLL_LAT * g.latency);
+            if (pl->flow_ready) {
+                // A flow task asks for all its cost rows at once, at most 24 per wave (they wait in
+                // registers), so its sources go on 1, 2 or 4 waves.  More waves shorten the task -- as long
+                // as the next layers' tasks still find room on the device beside the layer at work: the
+                // start of a task (four dependent round trips to memory before it reaches its gate) then
+                // lies behind it when its cost rows appear.  So: the most waves per task that keep two
+                // layers' tasks resident, else what keeps the most.  Measured (ms per solve, 1 / 2 / 4
+                // waves): S=22 V=16384 L=24 0.099 / 0.091 / 0.081; S=40 V=29493 L=28 - / 0.163 / 0.194.
+                auto waves_per_simd = [](int nsrc) { return nsrc <= 8 ? 6 : nsrc <= 12 ? 5 : nsrc <= 16 ? 4 : nsrc <= 20 ? 3 : 2; };
+                auto nsrc_for = [&](int K) {
+                    for (int c : GDP_FLOW_NSRC)
+                        if (c * K >= g.S) return c;
+                    return 0;
+                };
+                double band_tiles = 0;   // of an average layer, over the group
+                for (int k = g.first; k < g.first + g.count; ++k) band_tiles += (double)inst[(size_t)k].ntile * band_frac;
+                int best_K = 0;
+                double best_res = -1;
+                for (int K : {4, 2, 1}) {
+                    const int c = nsrc_for(K);
+                    if (!c) continue;
+                    const double res = (double)pl->num_cu * 4 * waves_per_simd(c) / std::max(1.0, band_tiles * g.ntb * K);
+                    if (res >= 2.0) { best_K = K; break; }
+                    if (res > best_res) { best_res = res; best_K = K; }
+                }
+                if (pl->latency_override >= 1 && nsrc_for(g.latency)) best_K = g.latency;
+                g.latency = best_K;
+                g.flow_nsrc = nsrc_for(best_K);
+                su = g.flow_nsrc * best_K;
+            }
+            g.lat_ok = su % (GDP_SRC_UNROLL_LAT * g.latency) == 0;
+            for (int k = g.first; k < g.first + g.count; ++k) inst[(size_t)k].SU = su;
         }
     }
     // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
@@ -1034,7 +1103,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         }
         // {tiles a reader reaches down, first tile to compute, last tile to compute} per layer
         h_band[(size_t)i].assign((size_t)h.L * 3, 0);
-        fill_bands(q, h, tile_rows, pl->skip, h_band[(size_t)i].data(), &pl->executed);
+        fill_bands(q, h, tile_rows, pl->skip, h_band[(size_t)i].data(), &pl->executed, pl->flow_ready);
         for (int k = 0; k < h.n_key; ++k) {
             GdpDevKey &key = dk[h.key_begin + k];
             key.other_mem = q->other_mem[k];
@@ -1074,9 +1143,24 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 y.m = d.M ? d.M + (int64_t)l * h.S * h.ldm : nullptr;
                 y.ld = h.ld; y.ldm = h.ldm;
                 y.S = h.S; y.SU = h.SU; y.SP = h.SP; y.ntile = h.ntile;
+                y.gate = 0;
+                if (pl->flow_ready && l >= 1)
+                    for (int part = 0; part < g.latency; ++part) {
+                        int best_s = 0, best_m = INT32_MAX;
+                        for (int u = 0; u < g.flow_nsrc; ++u) {
+                            const int s2 = part * g.flow_nsrc + u;
+                            if (s2 >= h.S) break;
+                            const int m = q->mem[(size_t)(l - 1) * h.S + s2];
+                            if (m < h.V && m < best_m) { best_m = m; best_s = u; }
+                        }
+                        y.gate |= (uint32_t)best_s << (8 * part);
+                    }
                 y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
                 y.lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
                 y.hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
+                if (y.hi >= y.lo)
+                    g.flow_blocks = std::max<int>(g.flow_blocks, (int)(((int64_t)(y.hi - y.lo + 1) * g.ntb * std::max(g.latency, 1) +
+                                                                         GDP_WAVES_PER_BLOCK - 1) / GDP_WAVES_PER_BLOCK));
                 if (y.hi >= y.lo)
                     g.live_blocks[(size_t)l] += ((int64_t)(y.hi - y.lo + 1) * g.ntb + GDP_WAVES_PER_BLOCK - 1) /
                                                 GDP_WAVES_PER_BLOCK;
@@ -1104,6 +1188,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 }
             }
             g.slots = (int)((widest + 7) / 8 * g.xcd_group);
+        }
+        if (const char *e = getenv("GALVATRON_DP_FLOW_WGS")) {
+            const int per_cu = atoi(e);
+            if (per_cu >= 1 && per_cu < 8 && pl->lds_per_cu >= 65536)
+                g.flow_lds = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
         sc->slots = g.slots;
         sc->spin_limit = pl->spin_limit;
@@ -1178,6 +1267,13 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                     64 * GDP_VARIANTS[g.variant].r,
                                     GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
+    }
+    if (pl->flow_ready) {
+        const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
+        for (const Group &g : pl->groups)
+            GDP_HIP(gdp_launch_flow_reset(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                          64 * GDP_VARIANTS[g.variant].r, g.sched.abort_flag, pl->stream));
+        pl->flow_clean = true;
     }
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
@@ -1333,13 +1429,24 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
         if (tasks / GDP_WAVES_PER_BLOCK + 16 > 0x7fffffffLL || g.count > 65535) return bad("grid of a per-layer launch", tasks, g.count, 0);
         if (g.latency && (g.latency != 1 && g.latency != 2 && g.latency != 4)) return bad("latency variant", g.latency, 0, 0);
         if (g.latency)
-            for (int k = 0; k < g.count; ++k)
-                if (pl->inst[(size_t)(g.first + k)].SU % (GDP_SRC_UNROLL_LAT * g.latency)) return bad("source padding of the latency variant", k, g.latency, 0);
+            for (int k = 0; k < g.count; ++k) {
+                const int su = pl->inst[(size_t)(g.first + k)].SU;
+                if (g.lat_ok && su % (GDP_SRC_UNROLL_LAT * g.latency)) return bad("source padding of the latency variant", k, g.latency, 0);
+                if (su % GDP_SRC_UNROLL) return bad("source padding", k, su, 0);
+                if (pl->flow_ready && (su != g.flow_nsrc * g.latency || su < g.S)) return bad("sources of a flow task", k, su, g.flow_nsrc);
+            }
     }
     return GDP_OK;
 }
 
 int run(gdp_plan *pl, int32_t mode, gdp_timing *t);
+
+size_t relax_launches(const gdp_plan *pl)
+{
+    size_t launches = 0;
+    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : pl->flow ? 1 : (size_t)g.max_L;
+    return launches;
+}
 
 // Everything of a run that does not wait: the launches and the copy of the results into the plan's
 // page-locked buffer, on the plan's stream.
@@ -1350,8 +1457,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     const GdpDevKey *d_keys = reinterpret_cast<const GdpDevKey *>(pl->dbase + pl->off_keys);
     GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
     int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
-    size_t launches = 0;
-    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : (size_t)g.max_L;
+    const size_t launches = relax_launches(pl);
     if (mode >= 2)
         while (pl->ev_relax.size() < 2 * launches) {
             hipEvent_t e;
@@ -1369,7 +1475,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                                         64 * GDP_VARIANTS[g.variant].r, what, pl->stream));
     }
     size_t li = 0;
-    if (pl->fused && !pl->holds_fused) {
+    if ((pl->fused || pl->flow) && !pl->holds_fused) {
         fused_turn_take();  // until run_finish has waited for the launch
         pl->holds_fused = true;
     }
@@ -1386,12 +1492,25 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
+    } else if (pl->flow) {
+        if (!pl->flow_clean)   // (plan creation and every flow run leave them clean; a run of another kind does not)
+            for (const Group &g : pl->groups)
+                GDP_HIP(gdp_launch_flow_reset(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                              64 * GDP_VARIANTS[g.variant].r, g.sched.abort_flag, pl->stream));
+        for (const Group &g : pl->groups) {
+            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
+            if (g.flow_blocks > 0)
+                GDP_HIP(gdp_launch_relax_flow(g.flow_nsrc, g.latency, g.sched.lay, g.max_L, g.count, g.flow_blocks, g.SP, 0, g.max_L,
+                                              g.sched.abort_flag, pl->spin_limit, g.flow_lds, pl->stream));
+            if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
+            ++li;
+        }
     } else {
         for (int l = 0; l < pl->max_L; ++l)
             for (const Group &g : pl->groups) {
                 if (l >= g.max_L) continue;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
-                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, pl->keep_marks ? 0 : g.latency,
+                GDP_HIP(gdp_launch_relax(g.variant, pl->keep_marks, pl->keep_marks || !g.lat_ok ? 0 : g.latency,
                                          reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
                                          g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
                 if (g.zero_layer[(size_t)l])
@@ -1404,6 +1523,20 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     if (mode >= 1) GDP_HIP(hipEventRecord(pl->ev_end, pl->stream));
     GDP_HIP(hipMemcpyAsync(pl->lane.back, pl->dbase + pl->off_abort, pl->back_bytes, hipMemcpyDeviceToHost,
                            pl->stream));
+    pl->wait_back = false;
+    pl->flow_clean = false;
+    bool exports = false;   // gdp_plan_fetch then reads the cost buffers: they are cleaned before the next run instead
+    for (const HostInst &h : pl->inst) exports = exports || (h.flags & (GDP_EXPORT_F | GDP_EXPORT_MARK));
+    if (pl->flow && !pl->one_shot && !exports) {
+        // NaN again into what the run wrote, behind the results: the caller does not wait for it, the
+        // next run on this stream (or the destruction of the plan) does
+        GDP_HIP(hipEventRecord(pl->lane.ev_back, pl->stream));
+        pl->wait_back = true;
+        for (const Group &g : pl->groups)
+            GDP_HIP(gdp_launch_flow_reset(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                          64 * GDP_VARIANTS[g.variant].r, g.sched.abort_flag, pl->stream));
+        pl->flow_clean = true;
+    }
     return GDP_OK;
 }
 
@@ -1411,9 +1544,8 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
 int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
 {
     GDP_HIP(hipSetDevice(pl->device));
-    size_t launches = 0;
-    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : (size_t)g.max_L;
-    const hipError_t waited = hipStreamSynchronize(pl->stream);
+    const size_t launches = relax_launches(pl);
+    const hipError_t waited = pl->wait_back ? hipEventSynchronize(pl->lane.ev_back) : hipStreamSynchronize(pl->stream);
     if (pl->holds_fused) {
         pl->holds_fused = false;
         fused_turn_give();
@@ -1422,12 +1554,13 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
     pl->h_out = reinterpret_cast<const GdpDevOut *>(pl->lane.back + (pl->off_out - pl->off_abort));
     pl->h_res = reinterpret_cast<const int32_t *>(pl->lane.back + (pl->off_res - pl->off_abort));
     // the flag is cleared and written by fused launches only
-    const int32_t aborted = pl->fused ? *reinterpret_cast<const int32_t *>(pl->lane.back) : 0;
+    const int32_t aborted = (pl->fused || pl->flow) ? *reinterpret_cast<const int32_t *>(pl->lane.back) : 0;
     if (aborted) {
         // Not every block of the fused launch was resident (the device is shared) or a wait ran out:
         // nothing of that run is kept; do the same work with one launch per layer instead.
         pl->ran = false;
         pl->fused = false;
+        pl->flow = false;
         pl->fused_gave_up = true;
         if (pl->no_fallback)
             return fail(GDP_E_HIP, "fused launch: a bounded wait ran out before its tiles were finished");
@@ -1441,12 +1574,13 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
         t->relax_bytes = pl->relax_bytes;
         t->relax_launches = (int32_t)launches;
         t->fused = pl->fused ? 1 : 0;
+        t->flow = pl->flow ? 1 : 0;
         if (!pl->groups.empty()) {
             const Group &g0 = pl->groups.front();
             t->tile_ts = GDP_VARIANTS[g0.variant].ts;
             t->tile_r = GDP_VARIANTS[g0.variant].r;
             t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
-            t->latency_variant = pl->fused ? 0 : g0.latency;
+            t->latency_variant = pl->fused || (!pl->flow && !g0.lat_ok) ? 0 : g0.latency;
         }
         t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));
@@ -1586,6 +1720,13 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
             if (value != 0 && !plan->can_fuse)
                 return fail(GDP_E_BADARG, "plan was laid out for per-layer launches only (two cost buffers, or a memory cost of 0)");
             plan->fused = value != 0;
+            plan->flow = false;
+            return GDP_OK;
+        case GDP_OPT_FLOW:
+            if (value != 0 && !plan->flow_ready)
+                return fail(GDP_E_BADARG, "plan was not laid out for a flow launch (see GALVATRON_DP_FLOW)");
+            plan->flow = value != 0;
+            if (plan->flow) plan->fused = false;
             return GDP_OK;
         case GDP_OPT_POISON:
             plan->poison = value != 0;
@@ -1676,6 +1817,7 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
         int rc = create_checked(end - begin, p + begin, &pl);
         int rp = prev ? run_finish(prev, 0, nullptr) : GDP_OK;
         if (rc == GDP_OK && rp == GDP_OK) {
+            pl->one_shot = true;
             rc = run_enqueue(pl, 0);
             if (rc != GDP_OK && pl->holds_fused) {
                 (void)hipStreamSynchronize(pl->stream);

@@ -77,7 +77,9 @@ struct GdpDevLayer {
     int64_t ld, ldm;    // elements per row of H / entries per row of M
     int32_t S, SU, SP, ntile;
     int32_t dep, lo, hi;  // see above; an entry of an instance without this layer has lo = 0, hi = -1
-    int32_t pad_[9];
+    uint32_t gate;        // flow launches: per part of a task (byte p for part p), the source strategy -- counted
+                          // within the part -- whose cost row lies highest (smallest memory cost in the layer before)
+    int32_t pad_[8];
     int64_t ro_head[16];  // copy of ro[0..16): a task that starts from them needs no second round trip
 };
 static_assert(sizeof(GdpDevLayer) == 256, "one record = four 64-byte scalar loads");
@@ -147,6 +149,21 @@ hipError_t gdp_launch_relax(int variant, bool marks, int latency, const GdpDevLa
 // With sched->rows set, layer0 is the first entry of that table and `layers` the number of entries.
 hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream);
+// (sources per wave, waves per task) of the flow kernels that are built
+#define GDP_FOR_EACH_FLOW(X) \
+    X(8, 1) X(12, 1) X(16, 1) X(20, 1) X(24, 1) X(8, 2) X(12, 2) X(16, 2) X(20, 2) X(24, 2) X(8, 4) X(12, 4) X(16, 4) X(20, 4) X(24, 4)
+static const int GDP_FLOW_NSRC[] = {8, 12, 16, 20, 24};
+// Layers layer0 .. layer0+layers-1 of the first n_inst instances of a group in one launch whose tasks
+// wait on the cost cells themselves (gdp_relax_flow_kernel; costs only, the tile of the latency variant,
+// `latency` = waves that share the sources of a task, nsrc = sources per wave: one of GDP_FLOW_NSRC, the
+// layers' SU being nsrc * latency).  grid_blocks: workgroups of the widest band.
+// The cells the launch writes must hold NaN beforehand and the abort flag zero: gdp_launch_flow_reset
+// (bands of all layers of n_inst instances).
+hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, unsigned lds_bytes,
+                                 hipStream_t stream);
+hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                                 int max_L, int tile_rows, int32_t *abort_flag, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);
 // GDP_INIT_ZERO: zeros in the data region of buffer 0 (the caller's initial f); GDP_INIT_POISON: NaN
 // in the data region of every other buffer (test aid: a read of a not-yet-written cell shows up);

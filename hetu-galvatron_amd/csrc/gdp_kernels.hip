@@ -291,6 +291,206 @@ __device__ __forceinline__ void relax_task_lat(const LatHead &H, unsigned tile, 
     }
 }
 
+// ---- tasks of a flow launch (gdp_relax_flow_kernel): waiting on the cost cells themselves --------------
+// lane_load at agent scope: the value comes from memory, never from a line that this XCD's L2 holds
+// from before another XCD wrote it.
+__device__ __forceinline__ double lane_load_agent(const double *row, unsigned lane_bytes)
+{
+    typedef const __attribute__((address_space(1))) char *gbytes;
+    typedef const __attribute__((address_space(1))) double *gdouble;
+    return __hip_atomic_load(
+        reinterpret_cast<gdouble>(reinterpret_cast<gbytes>(reinterpret_cast<uintptr_t>(row)) + lane_bytes),
+        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The abort flag of the launch, the number of polls after which a wave gives up, and what this wave
+// has used of it.  Every wait is bounded: a wave that has polled `limit` times, or finds the flag
+// raised, raises it and stops waiting (it finishes with whatever it reads; the host discards the run).
+struct FlowWait {
+    int32_t *abort_flag;
+    int64_t limit;
+    int64_t polls;
+    bool gave_up;
+};
+
+// One more poll: false when the wave has to stop waiting.  Sleeps a little first (waiting waves look
+// at single cells, one request per poll, so polling this often does not crowd the memory system).
+__device__ __forceinline__ bool flow_poll(FlowWait &w, unsigned lane)
+{
+    ++w.polls;
+    const int stop = (w.polls & 15) ? 0
+                                    : __builtin_amdgcn_readfirstlane(__hip_atomic_load(
+                                          w.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    if (w.polls > w.limit || stop != 0) {
+        if (lane == 0) __hip_atomic_store(w.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w.gave_up = true;
+        return false;
+    }
+    if (w.polls < 4) __builtin_amdgcn_s_sleep(1);
+    else __builtin_amdgcn_s_sleep(4);   // ~0.12 us
+    return true;
+}
+
+struct FlowHead {
+    const double *src, *it, *ia;
+    double *dst;
+    const int64_t *ro;
+    int64_t ld;
+    int S, SP, lo, hi;
+    unsigned gate;   // per part of a task (one byte each): the source, within the part, whose row lies highest
+};
+
+__device__ __forceinline__ FlowHead load_flow_head(const GdpDevLayer *Y)
+{
+    FlowHead h;
+    h.src = uload(&Y->src); h.dst = uload(&Y->dst); h.ro = uload(&Y->ro); h.it = uload(&Y->it);
+    h.ia = uload(&Y->ia); h.ld = uload(&Y->ld);
+    h.S = uload(&Y->S); h.SP = uload(&Y->SP); h.lo = uload(&Y->lo); h.hi = uload(&Y->hi);
+    h.gate = (unsigned)uload(&Y->gate);
+    // one round of scalar loads, all of it there before the first branch
+    asm volatile("" : "+s"(h.src), "+s"(h.dst), "+s"(h.ro), "+s"(h.it), "+s"(h.ia), "+s"(h.ld));
+    asm volatile("" : "+s"(h.S), "+s"(h.SP), "+s"(h.lo), "+s"(h.hi), "+s"(h.gate));
+    return h;
+}
+
+// One wave task of a flow launch: targets [tb*TS, tb*TS+TS) of the 64 rows of `tile`, against the NSRC
+// source strategies [part*NSRC, (part+1)*NSRC) (K parts per task, on K waves of the workgroup, as in
+// relax_task_lat; the layer's SU is NSRC*K).  Same arithmetic in the same order as relax_task, hence the
+// same bits.
+//   - What does not depend on the previous layer -- row offsets, the NSRC rows of transition costs (lane
+//     j of every row of 16 lanes holds column j), the intra costs -- is fetched first.
+//   - Then the task waits at a gate.  Before a run every cell that the run writes holds NaN, and no
+//     cost is ever NaN.  First one cell is asked for again and again (one request per poll) until it
+//     holds a cost: the highest cell the task reads (last row of the tile, source with the smallest
+//     memory cost), whose writer is the last to have been dispatched.  Then the first and the last cell
+//     of every one of the NSRC rows (one gathered load, lane u and lane NSRC + u for row u; the two
+//     can come from two tasks of the layer before), until all of them hold costs.
+//   - Then all NSRC cost rows are asked for at once, at agent scope, and consumed in order.  A row in which a lane still sees NaN (a task's stores need not show up
+//     together) is asked for again until it is whole.
+template <int TS, int NSRC, int K>
+__device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile, unsigned vtb, unsigned lane,
+                                                FlowWait &w)
+{
+    static_assert(K == 1 || GDP_WAVES_PER_BLOCK % K == 0, "parts of one task share a workgroup");
+    static_assert(TS <= 16, "a row of 16 lanes holds the transition costs of a step");
+    const unsigned tb = vtb / K, part = vtb % K;
+    const int SP = H.SP;
+    const double *src = H.src;
+    const int64_t *ro = H.ro + part * NSRC;
+    const int s0 = tb * TS;
+    const double *it = H.it + s0 + (int64_t)part * NSRC * SP;
+    const int64_t u0 = (int64_t)tile * 64;
+    unsigned lb = lane * 8u;
+    unsigned cb = ((lane & 15u) < (unsigned)TS ? (lane & 15u) : (unsigned)(TS - 1)) * 8u;
+    GDP_PIN_LANE(lb);
+    GDP_PIN_LANE(cb);
+
+    double best[1][TS];
+    int arg_unused[1][1];
+    double add_unused[TS];
+#pragma unroll
+    for (int j = 0; j < TS; ++j) { best[0][j] = INFINITY; add_unused[j] = 0.0; }
+
+    int64_t off[NSRC];
+#pragma unroll
+    for (int u = 0; u < NSRC; ++u) off[u] = uload(ro + u);
+    double scv[NSRC], iav;
+#pragma unroll
+    for (int u = 0; u < NSRC; ++u) {
+        const double *q = it + (int64_t)u * SP;
+        asm volatile("" : "+s"(q));
+        scv[u] = lane_load(q, cb, 0);
+    }
+    {
+        const double *qa = H.ia + s0;
+        asm volatile("" : "+s"(qa));
+        iav = lane_load(qa, cb, 0);
+    }
+    // the gate
+    {
+        static_assert(2 * NSRC <= 64, "one lane per end of a row");
+        const unsigned gu = lane < (unsigned)NSRC ? lane : lane < 2u * NSRC ? lane - NSRC : 0u;
+        const int64_t goff = ro[gu] + u0 + (lane >= (unsigned)NSRC ? 63 : 0);   // (a vector load of the row offsets)
+        const unsigned g1 = (H.gate >> (8u * part)) & 0xffu;
+        const double *cell1 = src + uload(ro + g1) + u0 + 63;
+        asm volatile("" : "+s"(cell1));
+        for (;;) {
+            const double y = lane_load_agent(cell1, 0u);
+            if (__builtin_amdgcn_ballot_w64(y != y) == 0) break;
+            if (!flow_poll(w, lane)) break;
+        }
+        // (asking for the rows right behind this load, without waiting for its answer, was slower:
+        // S=22 V=16384 L=24 0.099 -> 0.110 ms)
+        const double *cells = src + goff;
+        for (;;) {
+            double y = 0.0;
+            if (lane < 2u * NSRC) y = lane_load_agent(cells, 0u);
+            if (__builtin_amdgcn_ballot_w64(y != y) == 0) break;
+            if (w.gave_up || !flow_poll(w, lane)) break;
+        }
+    }
+    GDP_SCHED_FENCE();
+    double fp[NSRC][1];
+#pragma unroll
+    for (int u = 0; u < NSRC; ++u) {
+        fp[u][0] = lane_load_agent(src + off[u] + u0, lb);
+        GDP_SCHED_FENCE();
+    }
+#pragma unroll
+    for (int u = 0; u < NSRC; ++u) {
+        if (__builtin_amdgcn_ballot_w64(fp[u][0] != fp[u][0]) != 0) {
+            const double *row = src + uload(ro + u) + u0;   // (fetched again: the offsets are not kept in registers)
+            while (!w.gave_up && flow_poll(w, lane)) {
+                fp[u][0] = lane_load_agent(row, lb);
+                if (__builtin_amdgcn_ballot_w64(fp[u][0] != fp[u][0]) == 0) break;
+            }
+        }
+        double sc[TS];
+#pragma unroll
+        for (int j = 0; j < TS; ++j)   // lane j of every row of 16 lanes holds column j: one move spreads it
+            asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(sc[j]) : "v"(scv[u]), "n"(j));
+        relax_cols<TS, 1, false, 0, TS>(best, arg_unused, fp[u], sc, add_unused, u);
+        GDP_SCHED_FENCE();
+    }
+
+    bool mine[TS];
+#pragma unroll
+    for (int j = 0; j < TS; ++j) mine[j] = true;
+    if constexpr (K > 1) {
+        __shared__ double xch[GDP_WAVES_PER_BLOCK][TS][64];
+        const unsigned wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int j = 0; j < TS; ++j) xch[wv][j][lane] = best[0][j];
+        __syncthreads();   // waves of the workgroup that had no task have ended and are not waited for
+        const unsigned w0 = wv - part;   // the task's first wave
+#pragma unroll
+        for (int j = 0; j < TS; ++j) {
+            mine[j] = (unsigned)(j % K) == part;
+            if (mine[j]) {
+#pragma unroll
+                for (int pp = 0; pp < K; ++pp) best[0][j] = min_f64(best[0][j], xch[w0 + pp][j][lane]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < TS; ++j) {
+        double a;
+        asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(a) : "v"(iav), "n"(j));
+        best[0][j] += a;
+    }
+    const int64_t ld = H.ld;
+    const int nvalid = H.S - s0;
+    double *drow = H.dst + (int64_t)s0 * ld + u0;
+#pragma unroll
+    for (int j = 0; j < TS; ++j) {
+        if (j < nvalid) {
+            if (mine[j])
+                __hip_atomic_store(drow + lane, best[0][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            drow += ld;
+        }
+    }
+}
+
 // One wave task: targets [tb*TS, tb*TS+TS) of rows [tile*64*R, (tile+1)*64*R) of the layer described
 // by Y.
 // PUBLISH: the cost stores are write-through at agent scope, so that a wave on another XCD that
@@ -720,6 +920,60 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
                                __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- all layers in one launch, waiting on the cost cells themselves (small problems) ---------------
+// A problem whose layers are over in a few microseconds each spends its time between the layers: a
+// launch gap, the start of the workgroups, the first dependent loads; completion counters cost more
+// than they save at that size (a counter needs the stores acknowledged before it is bumped and a
+// round trip to be seen, before the first cost row can even be asked for).  Here the cost cells are
+// their own flags: before a run every cell that the run writes holds NaN (gdp_flow_reset_kernel) -- no
+// cost is ever NaN: NaN and -inf inputs are rejected on the host and +inf - inf cannot arise -- and a
+// task reads its cost rows at agent scope and asks again for any row in which a lane still sees NaN
+// (relax_task_flow).  A cell is one aligned 8-byte store, so a reader sees the pattern or the
+// cost, nothing in between; the stores are write-through at agent scope and nobody waits for them.
+// What a layer's task needs apart from the cost rows (its record, row offsets, transition and intra
+// costs) is fetched while the previous layer is still at work.
+// grid = (block tasks of the widest band, layers, instances): workgroups are dispatched in order of
+// their linear id, so every task a task waits for was dispatched before it (the argument of
+// gdp_relax_fused_kernel); waits are bounded, a wave that gives up raises the abort flag, the launch
+// drains and the host repeats the solve with one launch per layer.
+// The bands must be closed under reading: every row that a task of layer l's band reads from layer
+// l-1's output lies in that layer's band, below it (filled once per plan) or in the pads.
+template <int NSRC, int K>
+__global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 8 / GDP_WAVES_PER_BLOCK) void gdp_relax_flow_kernel(
+    const GdpDevLayer *__restrict__ lay, int max_L, int layer0, unsigned ntb, int32_t *abort_flag, int64_t spin_limit)
+{
+    const GdpDevLayer *Y = lay + ((int64_t)blockIdx.z * max_L + layer0 + (int)blockIdx.y);
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned lane = threadIdx.x & 63u;
+    const FlowHead H = load_flow_head(Y);
+    const unsigned live_tasks = H.hi >= H.lo ? (unsigned)(H.hi - H.lo + 1) * ntb : 0u;
+    const unsigned task = blockIdx.x * GDP_WAVES_PER_BLOCK + wave;   // ascending: what others wait for comes first
+    if (task >= live_tasks) return;
+    const unsigned t = task / ntb;
+    FlowWait fw = {abort_flag, spin_limit, 0, false};
+    relax_task_flow<GDP_LAT_TS, NSRC, K>(H, (unsigned)H.lo + t, task - t * ntb, lane, fw);
+}
+
+// NaN into every cell that a flow launch writes (the bands of all layers), and zero into its abort flag.
+// grid = (x chunks, rows 0..S-1, instances x layers); buffer l + 1 holds the output of layer l.
+__global__ __launch_bounds__(256) void gdp_flow_reset_kernel(const GdpDevInst *__restrict__ insts,
+                                                             const GdpDevLayer *__restrict__ lay, int max_L,
+                                                             int tile_rows, int32_t *abort_flag)
+{
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) *abort_flag = 0;
+    const int inst = blockIdx.z / max_L, l = blockIdx.z - inst * max_L;
+    const GdpDevInst *I = insts + inst;
+    if (l >= uload(&I->L) || (int)blockIdx.y >= uload(&I->S)) return;
+    const GdpDevLayer *Y = lay + ((int64_t)inst * max_L + l);
+    const int lo = uload(&Y->lo), hi = uload(&Y->hi);
+    if (hi < lo) return;
+    const int64_t first = (int64_t)lo * tile_rows, n = (int64_t)(hi - lo + 1) * tile_rows;
+    double *h = uload(&I->H) + (int64_t)(l + 1) * uload(&I->hstride) + (int64_t)blockIdx.y * uload(&I->ld) + uload(&I->P) + first;
+    const double nan = __builtin_nan("");
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        h[i] = nan;
+}
+
 __global__ __launch_bounds__(256) void gdp_zero_kernel(int32_t *p, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -1109,6 +1363,40 @@ hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched
         default: return hipErrorInvalidValue;
     }
 #undef X
+}
+
+hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, unsigned lds_bytes,
+                                 hipStream_t stream)
+{
+    if (n_inst < 1 || n_inst > 65535 || layers < 1 || layers > 65535 || grid_blocks < 1) return hipErrorInvalidValue;
+    const unsigned ntb = (unsigned)(SP / GDP_LAT_TS) * (unsigned)latency;  // with the parts of a split task
+    dim3 grid((unsigned)grid_blocks, (unsigned)layers, (unsigned)n_inst), block(64 * GDP_WAVES_PER_BLOCK);
+#define X(NSRC, K)                                                                                                   \
+    if (nsrc == NSRC && latency == K) {                                                                              \
+        hipLaunchKernelGGL((gdp_relax_flow_kernel<NSRC, K>), grid, block, lds_bytes, stream, lay, max_L, layer0, ntb, \
+                           abort_flag, spin_limit);                                                                  \
+        return hipGetLastError();                                                                                    \
+    }
+    GDP_FOR_EACH_FLOW(X)
+#undef X
+    return hipErrorInvalidValue;
+}
+
+hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                                 int max_L, int tile_rows, int32_t *abort_flag, hipStream_t stream)
+{
+    if (max_L < 1 || max_L > 65535 || n_inst < 1) return hipErrorInvalidValue;
+    unsigned bx = (unsigned)((max_ld + 256 * 8 - 1) / (256 * 8));
+    if (bx == 0) bx = 1;
+    if (bx > 64u) bx = 64u;
+    const int per = 65535 / max_L;  // instances per launch: grid.z holds at most 65535 (instance, layer) pairs
+    for (int i0 = 0; i0 < n_inst; i0 += per) {
+        const int n = n_inst - i0 < per ? n_inst - i0 : per;
+        hipLaunchKernelGGL(gdp_flow_reset_kernel, dim3(bx, (unsigned)max_S, (unsigned)(n * max_L)), dim3(256), 0, stream,
+                           insts + i0, lay + (int64_t)i0 * max_L, max_L, tile_rows, abort_flag);
+    }
+    return hipGetLastError();
 }
 
 hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)

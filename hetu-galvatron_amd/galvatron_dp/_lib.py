@@ -33,6 +33,7 @@ GDP_OPT_FUSED = 1
 GDP_OPT_SPIN_LIMIT = 2
 GDP_OPT_POISON = 3
 GDP_OPT_NO_FALLBACK = 4
+GDP_OPT_FLOW = 5
 
 GDP_STATIC_SCRATCH_BYTES = 64 << 20
 
@@ -72,7 +73,7 @@ class gdp_timing(ctypes.Structure):
                 ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("executed", ctypes.c_double),
                 ("relax_bytes", ctypes.c_double), ("tile_ts", ctypes.c_int32), ("tile_r", ctypes.c_int32),
                 ("keep_marks", ctypes.c_int32), ("chunk", ctypes.c_int32),
-                ("latency_variant", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("latency_variant", ctypes.c_int32), ("flow", ctypes.c_int32)]
 
 
 _lib = None

@@ -111,7 +111,7 @@ typedef struct gdp_timing {
     int32_t chunk;         /* instances taken through a fused launch together; 0: all, layer by layer */
     int32_t latency_variant; /* > 0: per-layer launches use the kernel variant for launches with few waves,
                                 with the source strategies of a task on this many waves (1, 2 or 4) */
-    int32_t reserved;
+    int32_t flow;          /* 1: all layers in one launch whose tasks wait on the cost cells themselves (small plans) */
 } gdp_timing;
 
 typedef struct gdp_plan gdp_plan;
@@ -171,6 +171,11 @@ void gdp_plan_destroy(gdp_plan *plan);
 #define GDP_OPT_SPIN_LIMIT 2
 #define GDP_OPT_POISON 3 /* test aid: NaN-fill every not-yet-written cost buffer before each run */
 #define GDP_OPT_NO_FALLBACK 4 /* test aid: an abandoned fused launch is an error, not a switch to per-layer */
+#define GDP_OPT_FLOW 5 /* 1: all layers in one launch whose tasks wait on the cost cells themselves: before a run
+                          every cell it writes holds NaN, a task reads its cost rows at agent scope and asks again
+                          for rows that are not whole yet.  Chosen by the library for plans too small for
+                          GDP_OPT_FUSED to pay (unless a launch scheme was asked for); only a plan laid out for it
+                          can be switched to 1.  0: one launch per layer.  Waits are bounded like GDP_OPT_FUSED's. */
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
 
 /* Frees the device allocations that finished plans left behind for reuse (no counterpart in the

@@ -172,6 +172,7 @@ def test_small_launches_use_the_latency_variant(S, monkeypatch):
                                      "GALVATRON_DP_FUSED", "GALVATRON_DP_LATENCY_VARIANT")):
         pytest.skip("the environment presets the layout")
     from oracle import dp_oracle as O
+    monkeypatch.setenv("GALVATRON_DP_FLOW", "0")     # (a plan this small would otherwise run all layers in one flow launch)
     rng = np.random.Generator(np.random.PCG64([3, S]))
     inst = W.random_instance(rng, 5, S, 700 + S, mem_hi=150, inf_frac=0.1, per_layer_inter=bool(S % 2), n_keys=3)
     wt, wr, wm, wf, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)

@@ -1,0 +1,159 @@
+"""GPU tests of the flow launch: all layers of a small plan in one launch whose tasks wait on the cost
+cells themselves (NaN = not written yet), through the C ABI.  Same bits as the oracle and as the
+reference-built goldens are required, as for every other launch scheme."""
+import os
+
+import numpy as np
+import pytest
+
+import helpers as H
+from galvatron_dp import _lib, workloads as W
+
+pytestmark = pytest.mark.gpu
+
+_PRESETS = ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R", "GALVATRON_DP_FUSED",
+            "GALVATRON_DP_LATENCY_VARIANT", "GALVATRON_DP_FLOW")
+
+
+def _problem(inst, **kw):
+    keys = sorted(inst.other_mem)
+    return _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                        [inst.other_time[k] for k in keys], inter_index=inst.inter_index, **kw)
+
+
+def _results(prob, keys):
+    return ({k: prob.total[i] for i, k in enumerate(keys)}, {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+            {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+
+
+def _check_against_golden(prob, rec, name):
+    keys = rec["keys"]
+    got = ({k: prob.total[i] for i, k in enumerate(keys)},
+           {k: [int(x) if prob.remaining[i] != -1 else -1 for x in prob.res[i]] for i, k in enumerate(keys)},
+           {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+    H.assert_same_results(got, H.golden_results(rec), name)
+
+
+@pytest.mark.parametrize("S", [1, 7, 8, 9, 12, 13, 22, 24, 25, 40, 44, 48, 49, 63, 96])
+def test_flow_launch_matches_the_oracle(S, monkeypatch):
+    """Small instances run as one flow launch by default; sources on 1, 2 and 4 waves per task where S
+    allows (S on both sides of every sources-per-wave step); f of the last layer compared too, and the
+    run repeated on the same plan (the cells are reset behind every run)."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    rng = np.random.Generator(np.random.PCG64([11, S]))
+    inst = W.random_instance(rng, 6, S, 900 + S, mem_hi=150, inf_frac=0.1, per_layer_inter=bool(S % 2), n_keys=3)
+    wt, wr, wm, wf, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+    keys = sorted(inst.other_mem)
+    seen = []
+    for preset in (None, "1", "2", "4"):
+        if preset is not None:
+            monkeypatch.setenv("GALVATRON_DP_LATENCY_VARIANT", preset)
+        for export_f in (False, True):
+            prob = _problem(inst, export_f=export_f)
+            with _lib.Plan([prob]) as plan:
+                for rep in range(3):
+                    if rep == 2:
+                        plan.set_option(_lib.GDP_OPT_POISON, 1)
+                    t = plan.run(1)
+                    plan.fetch()
+                    assert t.flow == 1 and t.fused == 0 and t.relax_launches == 1, (t.flow, t.fused, t.relax_launches)
+                    H.assert_same_results(_results(prob, keys), (wt, wr, wm), f"S={S} preset={preset} run {rep}")
+                    if export_f:
+                        assert prob.f_out.tobytes() == wf.tobytes()
+            seen.append(t.latency_variant)
+    for preset, k in zip(("1", "2", "4"), seen[2::2]):
+        if S <= 24 * int(preset):
+            assert k == int(preset), (preset, seen)
+
+
+def test_flow_launch_on_the_goldens(golden):
+    """cfg0 and the Galvatron-like instance at full size, with and without row skipping."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    for name in ("cfg0", "galvatron_like", "ties_6", "infeasible_9", "rand_5"):
+        rec = golden[name]
+        inst = H.build_case(rec)
+        for compute_all in (False, True):
+            prob = _problem(inst, compute_all=compute_all)
+            with _lib.Plan([prob]) as plan:
+                t = plan.run(1)
+                plan.fetch()
+                if name == "cfg0" or (name == "galvatron_like" and not compute_all):
+                    assert t.flow == 1
+                _check_against_golden(prob, rec, f"{name} compute_all={compute_all}")
+                t = plan.run(1)
+                plan.fetch()
+                _check_against_golden(prob, rec, f"{name} compute_all={compute_all} again")
+        prob = _problem(inst)
+        _lib.solve_batch([prob])
+        _check_against_golden(prob, rec, f"{name} solve")
+
+
+def test_flow_launch_batch_of_small_instances(golden, monkeypatch):
+    """Several small instances of different depth and S in one plan: one flow launch per group of equal S."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    monkeypatch.setenv("GALVATRON_DP_FLOW", "1")
+    names = ["ties_1", "rand_2", "cfg3_smallV_0", "infeasible_3", "rand_5", "cfg3_smallV_3", "ties_6", "rand_7"]
+    probs = [_problem(H.build_case(golden[n])) for n in names]
+    with _lib.Plan(probs) as plan:
+        for rep in range(2):
+            t = plan.run(1)
+            plan.fetch()
+            for n, prob in zip(names, probs):
+                _check_against_golden(prob, golden[n], f"{n} run {rep}")
+
+
+def test_flow_switched_off_and_on_again(golden):
+    """A plan laid out for the flow launch runs per layer when told to, and flows again afterwards (the
+    cells are reset first); a plan laid out for something else refuses the option."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    rec = golden["galvatron_like"]
+    inst = H.build_case(rec)
+    prob = _problem(inst)
+    with _lib.Plan([prob]) as plan:
+        for flow in (1, 0, 1, 1, 0, 0, 1):
+            plan.set_option(_lib.GDP_OPT_FLOW, flow)
+            t = plan.run(1)
+            plan.fetch()
+            assert t.flow == flow and t.fused == 0
+            assert t.relax_launches == (1 if flow else inst.L)
+            _check_against_golden(prob, rec, f"flow={flow}")
+    prob = _problem(inst, launch="per_layer")
+    with _lib.Plan([prob]) as plan:
+        t = plan.run(1)
+        assert t.flow == 0
+        with pytest.raises(ValueError):
+            plan.set_option(_lib.GDP_OPT_FLOW, 1)
+
+
+def test_abandoned_flow_launch_falls_back_or_reports(golden):
+    """A spin limit of 1 makes waiting wavefronts give up at once (forced from the host; every kernel
+    still runs to completion).  With the fallback the plan switches to per-layer launches and returns
+    the right answer; without it the run reports an error.  Either way the next plan works."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    rec = golden["cfg0"]
+    inst = H.build_case(rec)
+    prob = _problem(inst)
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_SPIN_LIMIT, 1)
+        t = plan.run(1)
+        plan.fetch()
+        _check_against_golden(prob, rec, "fallback")
+        assert t.flow == 0 and t.relax_launches == inst.L       # it did give up: 24 layers do not fit on the device at once
+        t = plan.run(1)
+        plan.fetch()
+        _check_against_golden(prob, rec, "after the fallback")
+    prob2 = _problem(inst)
+    with _lib.Plan([prob2]) as plan:
+        plan.set_option(_lib.GDP_OPT_SPIN_LIMIT, 1)
+        plan.set_option(_lib.GDP_OPT_NO_FALLBACK, 1)
+        with pytest.raises(RuntimeError, match="bounded wait"):
+            plan.run()
+    prob3 = _problem(inst)
+    _lib.solve_batch([prob3])
+    _check_against_golden(prob3, rec, "after")
