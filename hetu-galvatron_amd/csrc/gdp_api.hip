@@ -855,15 +855,50 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // instruction issue: their narrowest tile has a variant built for that (measured, 16 layers, one
     // instance: S=22 V=16384 0.176 -> 0.126 ms, S=44 V=16384 0.241 -> 0.208, S=64 V=4096 0.284 -> 0.192;
     // with all layers in one launch, or on larger problems, it is the slower one).
-    // Plans that small run all their layers in one launch that waits on the cost cells themselves
+    // Small and middling plans run all their layers in one launch that waits on the cost cells themselves
     // (gdp_relax_flow_kernel) -- unless the caller asked for a launch scheme: per-layer launches are also
-    // what a shared device wants, since they never wait.  GALVATRON_DP_FLOW=1 asks for it wherever the
-    // layout allows (costs only, no memory cost of 0, the tile of the latency variant).
+    // what a shared device wants, since they never wait.  A flow task asks for all its cost rows at once,
+    // at most 24 per wave (they wait in registers), so its sources go on 1, 2 or 4 waves.  More waves
+    // shorten the task -- as long as the next layers' tasks still find room on the device beside the layer
+    // at work: the start of a task (four dependent round trips to memory before it reaches its gate) then
+    // lies behind it when its cost rows appear.  So: the most waves per task that keep two layers' tasks
+    // resident, else what keeps the most (ms per solve, 1 / 2 / 4 waves: S=22 V=16384 L=24 0.099 / 0.091 /
+    // 0.081; S=40 V=29493 L=28 - / 0.163 / 0.194).  With less than 0.4 of a layer resident the launch with
+    // completion counters and wide tiles is the faster one (flow against it, by resident share: S=22 V=65536
+    // L=24, 1.0: 0.17 against 0.23 ms; S=44 V=32768 L=32, 0.5: 0.43 against 0.55; S=40 V=60000 L=28, 0.44:
+    // 0.44 against 0.49; S=44 V=65536 L=32, 0.25: 0.84 against 0.42).  GALVATRON_DP_FLOW=1 asks for it
+    // wherever the layout allows (costs only, no memory cost of 0, the tile of the latency variant).
+    struct FlowPick { int K, nsrc; double resident; };
+    auto flow_pick = [&](const Group &g) {
+        auto waves_per_simd = [](int nsrc) { return nsrc <= 8 ? 7 : nsrc <= 12 ? 6 : nsrc <= 16 ? 5 : nsrc <= 20 ? 4 : 3; };  // by their registers
+        auto nsrc_for = [&](int K) {
+            for (int c : GDP_FLOW_NSRC)
+                if (c * K >= g.S) return c;
+            return 0;
+        };
+        double band_tiles = 0;   // of an average layer, over the group
+        for (int k = g.first; k < g.first + g.count; ++k) band_tiles += (double)inst[(size_t)k].ntile * band_frac;
+        const int ntb8 = (g.S + GDP_LAT_TS - 1) / GDP_LAT_TS;
+        FlowPick best = {0, 0, -1.0};
+        for (int K : {4, 2, 1}) {
+            const int c = nsrc_for(K);
+            if (!c) continue;
+            const double res = (double)pl->num_cu * 4 * waves_per_simd(c) / std::max(1.0, band_tiles * ntb8 * K);
+            if (pl->latency_override >= 1 && K == (pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1))
+                return FlowPick{K, c, res};
+            if (res >= 2.0 && best.resident < 2.0) best = {K, c, res};
+            if (best.resident < 2.0 && res > best.resident) best = {K, c, res};
+        }
+        return best;
+    };
     bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused) : !fused_preset;
-    want_flow = want_flow && !pl->fused && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65535;
-    for (const Group &g : pl->groups)
+    want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65535;
+    for (const Group &g : pl->groups) {
         want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
+        if (want_flow && pl->flow_override != 1) want_flow = flow_pick(g).resident >= 0.4;
+    }
     pl->flow = pl->flow_ready = want_flow;
+    if (want_flow) pl->fused = false;
     for (Group &g : pl->groups) {
         const GdpVariant &v = GDP_VARIANTS[g.variant];
         bool on = !pl->fused && !pl->keep_marks && v.ts == GDP_LAT_TS && v.r == GDP_LAT_R;
@@ -884,34 +919,10 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             if (pl->latency_override >= 1) g.latency = pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1;
             int su = (int)align_up((size_t)g.S, (size_t)GDP_SRC_UNROLL_LAT * g.latency);
             if (pl->flow_ready) {
-                // A flow task asks for all its cost rows at once, at most 24 per wave (they wait in
-                // registers), so its sources go on 1, 2 or 4 waves.  More waves shorten the task -- as long
-                // as the next layers' tasks still find room on the device beside the layer at work: the
-                // start of a task (four dependent round trips to memory before it reaches its gate) then
-                // lies behind it when its cost rows appear.  So: the most waves per task that keep two
-                // layers' tasks resident, else what keeps the most.  Measured (ms per solve, 1 / 2 / 4
-                // waves): S=22 V=16384 L=24 0.099 / 0.091 / 0.081; S=40 V=29493 L=28 - / 0.163 / 0.194.
-                auto waves_per_simd = [](int nsrc) { return nsrc <= 8 ? 6 : nsrc <= 12 ? 5 : nsrc <= 16 ? 4 : nsrc <= 20 ? 3 : 2; };
-                auto nsrc_for = [&](int K) {
-                    for (int c : GDP_FLOW_NSRC)
-                        if (c * K >= g.S) return c;
-                    return 0;
-                };
-                double band_tiles = 0;   // of an average layer, over the group
-                for (int k = g.first; k < g.first + g.count; ++k) band_tiles += (double)inst[(size_t)k].ntile * band_frac;
-                int best_K = 0;
-                double best_res = -1;
-                for (int K : {4, 2, 1}) {
-                    const int c = nsrc_for(K);
-                    if (!c) continue;
-                    const double res = (double)pl->num_cu * 4 * waves_per_simd(c) / std::max(1.0, band_tiles * g.ntb * K);
-                    if (res >= 2.0) { best_K = K; break; }
-                    if (res > best_res) { best_res = res; best_K = K; }
-                }
-                if (pl->latency_override >= 1 && nsrc_for(g.latency)) best_K = g.latency;
-                g.latency = best_K;
-                g.flow_nsrc = nsrc_for(best_K);
-                su = g.flow_nsrc * best_K;
+                const FlowPick fp = flow_pick(g);
+                g.latency = fp.K;
+                g.flow_nsrc = fp.nsrc;
+                su = fp.nsrc * fp.K;
             }
             g.lat_ok = su % (GDP_SRC_UNROLL_LAT * g.latency) == 0;
             for (int k = g.first; k < g.first + g.count; ++k) inst[(size_t)k].SU = su;

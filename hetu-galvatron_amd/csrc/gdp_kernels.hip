@@ -394,14 +394,23 @@ __device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile
     int64_t off[NSRC];
 #pragma unroll
     for (int u = 0; u < NSRC; ++u) off[u] = uload(ro + u);
-    double scv[NSRC], iav;
-#pragma unroll
-    for (int u = 0; u < NSRC; ++u) {
-        const double *q = it + (int64_t)u * SP;
-        asm volatile("" : "+s"(q));
-        scv[u] = lane_load(q, cb, 0);
-    }
+    // The task's NSRC x TS transition costs wait in LDS, not in registers (registers decide how many
+    // tasks are resident, and the tasks of the next layer should be): each wave has a corner of its own,
+    // source-major, so that lane j of every row of 16 lanes reads column j of a step's row.
+    __shared__ double costs[GDP_WAVES_PER_BLOCK][NSRC * TS];
+    double *my_costs = costs[__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)];
+    double iav;
     {
+        static_assert(TS == 8, "eight lanes fetch a row of transition costs");
+#pragma unroll
+        for (int i0 = 0; i0 < NSRC * TS; i0 += 64) {
+            const unsigned i = (unsigned)i0 + lane;
+            if ((NSRC * TS) % 64 == 0 || i < (unsigned)(NSRC * TS)) {
+                const double *q = it;
+                asm volatile("" : "+s"(q));
+                my_costs[i] = lane_load(q, ((i >> 3) * (unsigned)SP + (i & 7u)) * 8u, 0);
+            }
+        }
         const double *qa = H.ia + s0;
         asm volatile("" : "+s"(qa));
         iav = lane_load(qa, cb, 0);
@@ -446,11 +455,11 @@ __device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile
             }
         }
         double sc[TS];
+        const double scv = my_costs[u * TS + (cb >> 3)];
 #pragma unroll
         for (int j = 0; j < TS; ++j)   // lane j of every row of 16 lanes holds column j: one move spreads it
-            asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(sc[j]) : "v"(scv[u]), "n"(j));
+            asm("v_mov_b64_dpp %0, %1 row_newbcast:%2 row_mask:0xf bank_mask:0xf" : "=v"(sc[j]) : "v"(scv), "n"(j));
         relax_cols<TS, 1, false, 0, TS>(best, arg_unused, fp[u], sc, add_unused, u);
-        GDP_SCHED_FENCE();
     }
 
     bool mine[TS];
