@@ -295,10 +295,12 @@ def main() -> int:
             "issued_per_relaxation": issued,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
             "bytes_per_launch": tm.relax_bytes / launches,
-            "scheme": "fused (all layers in one launch)" if tm.fused else "one launch per layer",
+            "scheme": ("fused (all layers in one launch)" if tm.fused else
+                       "flow (all layers in one launch, tasks wait on the cost cells themselves)" if tm.flow else
+                       "one launch per layer"),
             "tile": "%d target strategies x %d budget rows per wavefront" % (tm.tile_ts, 64 * tm.tile_r),
             "tile_key": "%dx%d" % (tm.tile_ts, tm.tile_r),
-            "kernel": "gdp_relax_fused_kernel" if tm.fused else
+            "kernel": "gdp_relax_fused_kernel" if tm.fused else "gdp_relax_flow_kernel" if tm.flow else
                       ("gdp_relax_kernel (latency variant)" if tm.latency_variant else "gdp_relax_kernel"),
             "clock_ghz": PROFILED_CLOCK_GHZ.get(workload) if compute_all and not keep_marks else None,
             "bit_exact": bit_exact,
