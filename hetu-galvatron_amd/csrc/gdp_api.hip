@@ -8,6 +8,7 @@
 #include "gdp_host.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -303,6 +304,17 @@ void fused_turn_take()
     g_fused_busy = true;
 }
 
+// The turn if it is free.  A flow plan that finds it taken does not queue up for it: it runs that solve
+// with one launch per layer, beside the launch that holds the turn (threads that call the plugin side by
+// side, as the reference's parallel search does, then overlap instead of taking turns).
+bool fused_turn_try_take()
+{
+    std::lock_guard<std::mutex> lk(g_fused_mu);
+    if (g_fused_busy) return false;
+    g_fused_busy = true;
+    return true;
+}
+
 void fused_turn_give()
 {
     {
@@ -444,6 +456,8 @@ struct gdp_plan {
     bool fused = true;            // one launch for all layers instead of one per layer
     bool flow = false;            // one launch for all layers whose tasks wait on the cost cells themselves (small
                                   // plans; see gdp_relax_flow_kernel); only with fused off
+    bool run_flow = false;        // the run in flight (or the last one) is a flow launch: a flow plan that does not
+                                  // get the turn runs that solve with one launch per layer
     bool flow_ready = false;      // the plan was laid out for it: closed bands, latency tile, NaN in the bands
     int flow_override = -1;       // GALVATRON_DP_FLOW=0|1: never / wherever the layout allows
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
@@ -1279,13 +1293,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                                     64 * GDP_VARIANTS[g.variant].r,
                                     GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
     }
-    if (pl->flow_ready) {
-        const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
-        for (const Group &g : pl->groups)
-            GDP_HIP(gdp_launch_flow_reset(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
-                                          64 * GDP_VARIANTS[g.variant].r, g.sched.abort_flag, pl->stream));
-        pl->flow_clean = true;
-    }
+    // (a plan laid out for the flow launch gets NaN into its bands when a run first takes that way: one that
+    // finds the turn taken every time never pays for it)
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);
@@ -1455,7 +1464,7 @@ int run(gdp_plan *pl, int32_t mode, gdp_timing *t);
 size_t relax_launches(const gdp_plan *pl)
 {
     size_t launches = 0;
-    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : pl->flow ? 1 : (size_t)g.max_L;
+    for (const Group &g : pl->groups) launches += pl->fused ? g.segments.size() : pl->run_flow ? 1 : (size_t)g.max_L;
     return launches;
 }
 
@@ -1468,6 +1477,17 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     const GdpDevKey *d_keys = reinterpret_cast<const GdpDevKey *>(pl->dbase + pl->off_keys);
     GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
     int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
+    pl->run_flow = false;
+    if (pl->fused && !pl->holds_fused) {
+        fused_turn_take();  // until run_finish has waited for the launch
+        pl->holds_fused = true;
+    } else if (pl->flow && !pl->fused) {
+        // (GALVATRON_DP_FLOW_WAIT=1: queue up for the turn like a fused plan does)
+        static const bool wait_turn = getenv("GALVATRON_DP_FLOW_WAIT") && atoi(getenv("GALVATRON_DP_FLOW_WAIT")) != 0;
+        if (pl->holds_fused) pl->run_flow = true;
+        else if (wait_turn) { fused_turn_take(); pl->holds_fused = pl->run_flow = true; }
+        else pl->holds_fused = pl->run_flow = fused_turn_try_take();
+    }
     const size_t launches = relax_launches(pl);
     if (mode >= 2)
         while (pl->ev_relax.size() < 2 * launches) {
@@ -1486,10 +1506,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                                         64 * GDP_VARIANTS[g.variant].r, what, pl->stream));
     }
     size_t li = 0;
-    if ((pl->fused || pl->flow) && !pl->holds_fused) {
-        fused_turn_take();  // until run_finish has waited for the launch
-        pl->holds_fused = true;
-    }
+
     if (pl->fused) {
         GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
                                 pl->stream));
@@ -1503,8 +1520,8 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
-    } else if (pl->flow) {
-        if (!pl->flow_clean)   // (plan creation and every flow run leave them clean; a run of another kind does not)
+    } else if (pl->run_flow) {
+        if (!pl->flow_clean)   // (every flow run of a plan that runs again leaves them clean; nothing else does)
             for (const Group &g : pl->groups)
                 GDP_HIP(gdp_launch_flow_reset(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                               64 * GDP_VARIANTS[g.variant].r, g.sched.abort_flag, pl->stream));
@@ -1538,7 +1555,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     pl->flow_clean = false;
     bool exports = false;   // gdp_plan_fetch then reads the cost buffers: they are cleaned before the next run instead
     for (const HostInst &h : pl->inst) exports = exports || (h.flags & (GDP_EXPORT_F | GDP_EXPORT_MARK));
-    if (pl->flow && !pl->one_shot && !exports) {
+    if (pl->run_flow && !pl->one_shot && !exports) {
         // NaN again into what the run wrote, behind the results: the caller does not wait for it, the
         // next run on this stream (or the destruction of the plan) does
         GDP_HIP(hipEventRecord(pl->lane.ev_back, pl->stream));
@@ -1565,7 +1582,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
     pl->h_out = reinterpret_cast<const GdpDevOut *>(pl->lane.back + (pl->off_out - pl->off_abort));
     pl->h_res = reinterpret_cast<const int32_t *>(pl->lane.back + (pl->off_res - pl->off_abort));
     // the flag is cleared and written by fused launches only
-    const int32_t aborted = (pl->fused || pl->flow) ? *reinterpret_cast<const int32_t *>(pl->lane.back) : 0;
+    const int32_t aborted = (pl->fused || pl->run_flow) ? *reinterpret_cast<const int32_t *>(pl->lane.back) : 0;
     if (aborted) {
         // Not every block of the fused launch was resident (the device is shared) or a wait ran out:
         // nothing of that run is kept; do the same work with one launch per layer instead.
@@ -1585,13 +1602,13 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
         t->relax_bytes = pl->relax_bytes;
         t->relax_launches = (int32_t)launches;
         t->fused = pl->fused ? 1 : 0;
-        t->flow = pl->flow ? 1 : 0;
+        t->flow = pl->run_flow ? 1 : 0;
         if (!pl->groups.empty()) {
             const Group &g0 = pl->groups.front();
             t->tile_ts = GDP_VARIANTS[g0.variant].ts;
             t->tile_r = GDP_VARIANTS[g0.variant].r;
             t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
-            t->latency_variant = pl->fused || (!pl->flow && !g0.lat_ok) ? 0 : g0.latency;
+            t->latency_variant = pl->fused || (!pl->run_flow && !g0.lat_ok) ? 0 : g0.latency;
         }
         t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));

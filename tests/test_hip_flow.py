@@ -157,3 +157,40 @@ def test_abandoned_flow_launch_falls_back_or_reports(golden):
     prob3 = _problem(inst)
     _lib.solve_batch([prob3])
     _check_against_golden(prob3, rec, "after")
+
+
+def test_flow_plans_from_several_threads(golden):
+    """Threads that call the plugin side by side (as the reference's parallel search does): one flow
+    launch runs at a time, a plan that finds the turn taken solves with one launch per layer beside
+    it.  Every result equals the reference's, whichever way a call ran."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    import threading
+    names = ["cfg0", "galvatron_like", "rand_5", "ties_6"]
+    errors, flowed = [], []
+
+    def work(tid):
+        try:
+            for it in range(12):
+                name = names[(tid + it) % len(names)]
+                rec = golden[name]
+                prob = _problem(H.build_case(rec))
+                if it % 2:
+                    _lib.solve_batch([prob])
+                else:
+                    with _lib.Plan([prob]) as plan:
+                        for _ in range(3):
+                            flowed.append(plan.run(1).flow)
+                            plan.fetch()
+                            _check_against_golden(prob, rec, f"thread {tid} {name}")
+                _check_against_golden(prob, rec, f"thread {tid} {name}")
+        except Exception as e:       # noqa: BLE001
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert any(flowed)
