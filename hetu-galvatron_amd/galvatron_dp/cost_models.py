@@ -450,11 +450,29 @@ def memory_cost_rows(strategies, global_batch_size, mbsz, min_tp, max_tp, stage_
     else:
         activation = plain
 
-    s0 = strategies[0]
-    z2, z3 = _zero_ratios(int(chunks[0]), train_args.mixed_precision, train_args.async_grad_reduce)
-    other = _other_memory(s0, int(chunks[0]), z2, z3, global_batch_size, min_tp, max_tp, vsp, embed_sdp, train_args,
-                          parallel_args, profile_model_args)
+    other = memory_cost_other(strategies, global_batch_size, mbsz, min_tp, max_tp, vsp=vsp, embed_sdp=embed_sdp,
+                              model_args=model_args, train_args=train_args, parallel_args=parallel_args,
+                              profile_model_args=profile_model_args)
     return states + activation, other
+
+
+def memory_cost_other(strategies, global_batch_size, mbsz, min_tp, max_tp, vsp=0, embed_sdp=False, model_args=None,
+                      train_args=None, parallel_args=None, profile_model_args=None):
+    """The ``'other'`` entry of ``MemoryCostModel(strategies[0], ...).get_memory_cost()`` alone -- the one
+    part of ``memory_cost_rows`` that depends on ``max_tp``, ``vsp`` and ``embed_sdp`` (the per-layer
+    rows do not, so a sweep can keep them while it walks through those).  For inputs that
+    ``memory_cost_rows`` accepts."""
+    s0 = strategies[0]
+    asked = parallel_args.chunks
+    if asked is None:
+        asked = float(parallel_args.optimal_chunk_func(global_batch_size // s0[2], s0, mbsz, min_tp))
+    cap = global_batch_size // (int(s0[1]) * int(s0[2]) // min_tp)
+    if cap == 0:
+        cap = 1
+    chunks0 = int(cap if asked > cap else asked)                           # int() of the class: towards zero
+    z2, z3 = _zero_ratios(chunks0, train_args.mixed_precision, train_args.async_grad_reduce)
+    return _other_memory(s0, chunks0, z2, z3, global_batch_size, min_tp, max_tp, vsp, embed_sdp, train_args,
+                         parallel_args, profile_model_args)
 
 
 # ---- time -------------------------------------------------------------------------------------------

@@ -272,6 +272,10 @@ class DpOnModel:
             self.max_mem -= self.mem_cache
         self.model_microbatch_after_dp = model_microbatch_after_dp
         self.pipeline_type = pipeline_type
+        # Optional (no counterpart in the reference): a dict shared by the DpOnModel objects of one sweep,
+        # which all hold the SAME strategy lists and argument records.  Rows of intra-layer times are
+        # then computed once per (strategies, batch size, layer type) instead of once per task.
+        self.row_cache = None
 
     def match_strategy(self, s1, s2, except_keys=[]):
         return _same_strategy(s1, s2, tuple(except_keys))
@@ -289,6 +293,16 @@ class DpOnModel:
         for i, n in enumerate(self.layer_num):
             b = bsz / chunks[i] if self.model_microbatch_after_dp else bsz
             row = None
+            key = None
+            if self.row_cache is not None:
+                # the strategy lists and records are the sweep's own objects (kept alive by the entry)
+                key = ("time", tuple(map(id, strategy_set)), b, i, id(self.timecost_model),
+                       id(self.profile_hardware_args_list[i]), id(self.model_args_list[i]), id(self.train_args_list[i]),
+                       id(self.parallel_args_list[i]), id(self.profile_model_args_list[i]))
+                hit = self.row_cache.get(key)
+                if hit is not None:
+                    blocks.append(hit[0].reshape(1, -1).repeat(n, axis=0))
+                    continue
             if self.timecost_model is cost_models.TimeCostModel:
                 try:
                     row = cost_models.time_cost_rows(strategy_set, b,
@@ -299,7 +313,11 @@ class DpOnModel:
             if row is None:
                 row = [self.timecost_model(s, b, profile_hardware_args=self.profile_hardware_args_list[i],
                                            logger=self.logger, **self._model_kwargs(i)).gen_result() for s in strategy_set]
-            blocks.append(np.array(row, dtype=np.float64).reshape(1, -1).repeat(n, axis=0))
+            row = np.array(row, dtype=np.float64)
+            if key is not None:
+                self.row_cache[key] = (row, list(strategy_set), self.profile_hardware_args_list[i], self.model_args_list[i],
+                                       self.train_args_list[i], self.parallel_args_list[i], self.profile_model_args_list[i])
+            blocks.append(row.reshape(1, -1).repeat(n, axis=0))
         return np.concatenate(blocks, axis=0)
 
     def _memory_rows(self, strategy_set, i, bsz, mbsz, min_tp, max_tp, vsp, embed_sdp, stage_ids):
@@ -307,10 +325,25 @@ class DpOnModel:
         ``i``: one array evaluation with this package's own memory model, one object per strategy and
         stage otherwise.  ``stage_ids`` is ``[None]`` where the stage does not matter (gpipe)."""
         if self.memcost_model is cost_models.MemoryCostModel:
+            key = None
+            if self.row_cache is not None:
+                # the rows depend on neither max_tp nor vsp nor embed_sdp: a sweep that walks through those
+                # keeps them and recomputes the 'other' entry alone
+                key = ("mem", tuple(map(id, strategy_set)), bsz, mbsz, min_tp, tuple(stage_ids), i,
+                       id(self.model_args_list[i]), id(self.train_args_list[i]), id(self.parallel_args_list[i]),
+                       id(self.profile_model_args_list[i]))
+                hit = self.row_cache.get(key)
+                if hit is not None:
+                    other = cost_models.memory_cost_other(strategy_set, bsz, mbsz, min_tp, max_tp, vsp=vsp,
+                                                          embed_sdp=embed_sdp, **self._model_kwargs(i)) if i == 0 else None
+                    return hit[0], other
             try:
                 rows, other = cost_models.memory_cost_rows(
                     strategy_set, bsz, mbsz, min_tp, max_tp, vsp=vsp, embed_sdp=embed_sdp,
                     stage_idx=[0 if x is None else x for x in stage_ids], **self._model_kwargs(i))
+                if key is not None:
+                    self.row_cache[key] = (rows, list(strategy_set), self.model_args_list[i], self.train_args_list[i],
+                                           self.parallel_args_list[i], self.profile_model_args_list[i])
                 return rows, other
             except cost_models.NotVectorisable:
                 pass
@@ -369,6 +402,13 @@ class DpOnModel:
         [1 + layer types, S, S] -- matrix 0 is all zeros, for the first layer of the model, which has no
         switch before it (dynamic_programming.py:372) -- and ``index`` [L] naming every layer's matrix."""
         S = len(strategy_set)
+        key = None
+        if self.row_cache is not None:
+            key = ("inter", tuple(map(id, strategy_set)), mbsz, min_tp, id(self.comm_coe_dict), id(self.config),
+                   tuple(self.sequence_len), tuple(self.layer_num))
+            hit = self.row_cache.get(key)
+            if hit is not None:
+                return hit[0], hit[1]
         tables = np.zeros((1 + len(self.layer_num), S, S), dtype=np.float64)
         index = []
         for idx, n in enumerate(self.layer_num):
@@ -376,6 +416,8 @@ class DpOnModel:
             index += [1 + idx] * n
         index = np.array(index, dtype=np.int32)
         index[0] = 0
+        if key is not None:
+            self.row_cache[key] = (tables, index, list(strategy_set), self.comm_coe_dict, self.config)
         return tables, index
 
     def _inter_cost(self, strategy_set, mbsz, min_tp):

@@ -77,6 +77,8 @@ class SearchEngine:
         self.optimal = None
         self.solved_instances = 0
         self.keep_device_cache = False      # True: a sweep leaves the library's cached device allocations in place
+        self.overlap_part = 512             # DP instances per part handed to the device while later tasks are still
+                                            # being prepared on the host; 0: one batch when everything is prepared
 
     # ---- model, paths (search_engine.py:45-97) ---------------------------------------------------------
     def set_model(self, model_name, model_layer_configs, path=None):
@@ -392,6 +394,16 @@ class SearchEngine:
         self.strategies = copy.deepcopy(self.strategies)
         pending = []               # (task, sp_search, DpOnModel, ticket, first instance, number of instances, stage)
         all_dps = []
+        row_cache = {}             # intra-layer time rows, shared by the DpOnModel objects of this sweep
+        # The device solves what has been prepared so far while the next tasks are being prepared: the
+        # instances go to a worker thread in parts of at least `part` (the library call releases the
+        # interpreter lock while the device works).
+        part = self.overlap_part if one_batch else 0
+        solved, sent = [], 0       # futures of the parts, instances handed over so far
+        pool = None
+        if part:
+            from concurrent.futures import ThreadPoolExecutor
+            pool = ThreadPoolExecutor(1)
         for task in self.tasks():
             bsz, chunk, min_tp, max_tp, vsp, embed_sdp = task
             for sp_search in sp_searches:
@@ -402,12 +414,25 @@ class SearchEngine:
                     continue
                 cand, mbsz, stage = picked
                 model = self._dp_on_model(cand, stage)
+                model.row_cache = row_cache
                 check_optimal_chunks(self.args.gpu_num, cand, self.optimal_chunk_func, bsz, mbsz, min_tp)
                 ticket, dps = model.fit_begin(bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, mbsz_dict=mbsz)
                 pending.append((task, sp_search, model, ticket, len(all_dps), len(dps), stage))
                 all_dps += dps
+                if pool is not None and len(all_dps) - sent >= part:
+                    solved.append(pool.submit(DPAlg.fit_many, all_dps[sent:]))
+                    sent = len(all_dps)
         self.solved_instances = len(all_dps)
-        if one_batch:
+        if pool is not None:
+            try:
+                if sent < len(all_dps):
+                    solved.append(pool.submit(DPAlg.fit_many, all_dps[sent:]))
+                fits = []
+                for f in solved:
+                    fits += f.result()
+            finally:
+                pool.shutdown(wait=True)
+        elif one_batch:
             fits = DPAlg.fit_many(all_dps)
         else:
             fits = []
