@@ -906,7 +906,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         return best;
     };
     bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused) : !fused_preset;
-    want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65535;
+    want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65534;
     for (const Group &g : pl->groups) {
         want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
         if (want_flow && pl->flow_override != 1) want_flow = flow_pick(g).resident >= 0.4;
@@ -1180,6 +1180,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                         }
                         y.gate |= (uint32_t)best_s << (8 * part);
                     }
+                // Rows of this layer's output below its band are +inf and are filled once per plan -- those that
+                // something reads: the band of the next layer reaches down by at most this layer's largest
+                // memory cost (the backtrack reads what the relaxation read), the epilogue and the pass for
+                // memory costs of 0 read anywhere.
+                y.fill_from = 0;
+                if (l + 1 < h.L && !h.has_zero) {
+                    const int64_t lo_next = h_band[(size_t)(g.first + k)][3 * (size_t)(l + 1) + 1];
+                    const int64_t reach = (int64_t)h_band[(size_t)(g.first + k)][3 * (size_t)l];   // tiles
+                    y.fill_from = (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
+                }
                 y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
                 y.lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
                 y.hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
@@ -1288,13 +1298,25 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
-        for (const Group &g : pl->groups)
-            GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
-                                    64 * GDP_VARIANTS[g.variant].r,
-                                    GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
+        // A plan laid out for the flow launch gets NaN into its bands here if the turn is free right now (its
+        // first run will most likely flow), else when a run first takes that way: a plan that finds the turn
+        // taken every time never pays for it.
+        bool nan_bands = false;
+        if (pl->flow_ready) {
+            std::lock_guard<std::mutex> lk(g_fused_mu);
+            nan_bands = !g_fused_busy;
+        }
+        for (const Group &g : pl->groups) {
+            if (!nan_bands)   // (one launch instead of three pays only where the three are short)
+                GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                        64 * GDP_VARIANTS[g.variant].r,
+                                        GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
+            else
+                GDP_HIP(gdp_launch_prepare(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
+                                           64 * GDP_VARIANTS[g.variant].r, nan_bands, g.sched.abort_flag, pl->stream));
+        }
+        pl->flow_clean = nan_bands;
     }
-    // (a plan laid out for the flow launch gets NaN into its bands when a run first takes that way: one that
-    // finds the turn taken every time never pays for it)
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);

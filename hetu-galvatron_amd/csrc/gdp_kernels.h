@@ -79,7 +79,9 @@ struct GdpDevLayer {
     int32_t dep, lo, hi;  // see above; an entry of an instance without this layer has lo = 0, hi = -1
     uint32_t gate;        // flow launches: per part of a task (byte p for part p), the source strategy -- counted
                           // within the part -- whose cost row lies highest (smallest memory cost in the layer before)
-    int32_t pad_[8];
+    int32_t fill_from;    // first row of this layer's output below its band that anything reads (rows fill_from ..
+                          // lo * tile rows - 1 are filled with +inf once per plan; the rows below are never touched)
+    int32_t pad_[7];
     int64_t ro_head[16];  // copy of ro[0..16): a task that starts from them needs no second round trip
 };
 static_assert(sizeof(GdpDevLayer) == 256, "one record = four 64-byte scalar loads");
@@ -170,6 +172,10 @@ hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t ma
 // GDP_INIT_FILL (one cost buffer per layer only): +inf in the rows of layer l's output below its
 // first tile with arithmetic, lay[i * max_L + l].lo (every source cell of those rows is +inf, so the
 // cells are +inf whatever the costs: written once per plan, the costs-only kernels leave them alone).
+// GDP_INIT_PADS | GDP_INIT_ZERO | GDP_INIT_FILL of a costs-only plan (one cost buffer per layer) in one
+// launch, and, with nan_bands, what gdp_launch_flow_reset does as well.
+hipError_t gdp_launch_prepare(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                              int max_L, int tile_rows, bool nan_bands, int32_t *abort_flag, hipStream_t stream);
 #define GDP_INIT_PADS 1
 #define GDP_INIT_ZERO 2
 #define GDP_INIT_POISON 4

@@ -998,11 +998,56 @@ __global__ __launch_bounds__(256) void gdp_fill_kernel(const GdpDevInst *__restr
     const GdpDevInst *I = insts + inst;
     if (l >= uload(&I->L) || (int)blockIdx.y >= uload(&I->S)) return;
     int64_t n = (int64_t)uload(&lay[(int64_t)inst * max_L + l].lo) * tile_rows;
+    const int64_t from = uload(&lay[(int64_t)inst * max_L + l].fill_from);
     const int64_t ldm = uload(&I->ldm);
     if (n > ldm) n = ldm;
     double *h = uload(&I->H) + (int64_t)(l + 1) * uload(&I->hstride) + (int64_t)blockIdx.y * uload(&I->ld) + uload(&I->P);
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    for (int64_t i = from + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
         h[i] = INFINITY;
+}
+
+// Everything a costs-only plan needs in its cost buffers before its first run, in one launch: +inf in
+// the pads in front of every row and in the +inf row of every buffer, zeros in buffer 0 (the caller's
+// initial f), +inf in the rows below the band of every layer's output that something reads, and -- with
+// `nan_bands`, for a plan that will run as a flow launch -- NaN in the bands.
+// grid = (x chunks, rows 0..S, instances x (max_L + 1) buffers).
+__global__ __launch_bounds__(256) void gdp_prepare_kernel(const GdpDevInst *__restrict__ insts,
+                                                          const GdpDevLayer *__restrict__ lay, int max_L, int tile_rows,
+                                                          int nan_bands, int32_t *abort_flag)
+{
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) *abort_flag = 0;
+    const int inst = blockIdx.z / (max_L + 1), b = blockIdx.z - inst * (max_L + 1);
+    const GdpDevInst *I = insts + inst;
+    const int S = uload(&I->S), L = uload(&I->L);
+    const int row = blockIdx.y;
+    if (b > L || row > S) return;
+    const int64_t ld = uload(&I->ld);
+    const int64_t P = uload(&I->P);
+    double *h = uload(&I->H) + (int64_t)b * uload(&I->hstride) + (int64_t)row * ld;
+    int64_t fill_from = 0, band_from = 0, band_to = 0;   // rows of this buffer (layer b - 1's output)
+    if (b >= 1) {
+        const GdpDevLayer *Y = lay + ((int64_t)inst * max_L + (b - 1));
+        const int lo = uload(&Y->lo), hi = uload(&Y->hi);
+        fill_from = uload(&Y->fill_from);
+        band_from = (int64_t)lo * tile_rows;
+        band_to = hi >= lo ? (int64_t)(hi + 1) * tile_rows : band_from;
+        if (band_from > ld - P) band_from = ld - P;
+        if (band_to > ld - P) band_to = ld - P;
+    }
+    const double inf = INFINITY;
+    const double nan = __builtin_nan("");
+    if (row == S || b == 0) {   // the whole row
+        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ld; i += (int64_t)gridDim.x * blockDim.x)
+            h[i] = (row == S || i < P) ? inf : 0.0;
+        return;
+    }
+    // the pad, then rows fill_from .. end of what is written (nothing in between is touched)
+    const int64_t end = nan_bands ? band_to : band_from;
+    const int64_t n = P + (end > fill_from ? end - fill_from : 0);
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t u = j < P ? j - P : j - P + fill_from;
+        h[P + u] = (u < band_from) ? inf : nan;
+    }
 }
 
 __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts, int what)
@@ -1414,6 +1459,22 @@ hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream)
     unsigned nb = (unsigned)((n + 1023) / 1024);
     if (nb > 4096u) nb = 4096u;
     hipLaunchKernelGGL(gdp_zero_kernel, dim3(nb), dim3(256), 0, stream, p, n);
+    return hipGetLastError();
+}
+
+hipError_t gdp_launch_prepare(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
+                              int max_L, int tile_rows, bool nan_bands, int32_t *abort_flag, hipStream_t stream)
+{
+    if (max_L < 1 || max_L > 65534 || n_inst < 1) return hipErrorInvalidValue;
+    unsigned bx = (unsigned)((max_ld + 256 * 4 - 1) / (256 * 4));
+    if (bx == 0) bx = 1;
+    if (bx > 64u) bx = 64u;
+    const int per = 65535 / (max_L + 1);  // instances per launch: grid.z holds at most 65535 (instance, buffer) pairs
+    for (int i0 = 0; i0 < n_inst; i0 += per) {
+        const int n = n_inst - i0 < per ? n_inst - i0 : per;
+        hipLaunchKernelGGL(gdp_prepare_kernel, dim3(bx, (unsigned)(max_S + 1), (unsigned)(n * (max_L + 1))), dim3(256), 0,
+                           stream, insts + i0, lay + (int64_t)i0 * max_L, max_L, tile_rows, nan_bands ? 1 : 0, abort_flag);
+    }
     return hipGetLastError();
 }
 
