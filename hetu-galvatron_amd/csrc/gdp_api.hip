@@ -185,6 +185,8 @@ struct Lane {
     hipStream_t stream = nullptr;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     hipEvent_t ev_back = nullptr;  // after the copy of the results (a flow run queues more work behind it)
+    hipStream_t side = nullptr;    // second stream: the upload of a small plan's inputs runs beside the kernel that
+    hipEvent_t ev_side = nullptr;  // prepares its cost buffers; the event joins it to the main stream
     char *back = nullptr;  // page-locked host memory the results are copied into
     size_t back_bytes = 0;
     char *up = nullptr;    // page-locked host memory the inputs' device layout is built in (may be absent)
@@ -199,6 +201,8 @@ void lane_release(Lane &ln)  // the lane's device is current
     if (ln.ev_begin) (void)hipEventDestroy(ln.ev_begin);
     if (ln.ev_end) (void)hipEventDestroy(ln.ev_end);
     if (ln.ev_back) (void)hipEventDestroy(ln.ev_back);
+    if (ln.ev_side) (void)hipEventDestroy(ln.ev_side);
+    if (ln.side) (void)hipStreamDestroy(ln.side);
     if (ln.stream) (void)hipStreamDestroy(ln.stream);
     if (ln.back) (void)hipHostFree(ln.back);
     if (ln.up) (void)hipHostFree(ln.up);
@@ -242,6 +246,8 @@ hipError_t lane_take(int device, size_t back_bytes, size_t up_bytes, Lane *out)
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_begin);
         if (e == hipSuccess) e = hipEventCreate(&ln.ev_end);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&ln.ev_back, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipStreamCreateWithFlags(&ln.side, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&ln.ev_side, hipEventDisableTiming);
     }
     if (e == hipSuccess) e = pinned_reserve(&ln.back, &ln.back_bytes, back_bytes, 65536);
     if (e == hipSuccess && up_bytes <= UPLOAD_PINNED_MAX) e = pinned_reserve(&ln.up, &ln.up_bytes, up_bytes, (size_t)1 << 20);
@@ -456,6 +462,7 @@ struct gdp_plan {
     bool fused = true;            // one launch for all layers instead of one per layer
     bool flow = false;            // one launch for all layers whose tasks wait on the cost cells themselves (small
                                   // plans; see gdp_relax_flow_kernel); only with fused off
+    bool split_upload = false;    // the per-instance inputs were uploaded on the lane's second stream
     bool run_flow = false;        // the run in flight (or the last one) is a flow launch: a flow plan that does not
                                   // get the turn runs that solve with one launch per layer
     bool flow_ready = false;      // the plan was laid out for it: closed bands, latency tile, NaN in the bands
@@ -581,6 +588,7 @@ void destroy(gdp_plan *pl)
     }
     if (pl->dbase || pl->lane.stream) (void)hipSetDevice(pl->device);
     if (pl->lane.stream) (void)hipStreamSynchronize(pl->lane.stream);  // the upload may still read its host copy
+    if (pl->split_upload && pl->lane.side) (void)hipStreamSynchronize(pl->lane.side);   // (joined to the main stream: idle by now)
     if (pl->holds_fused) {  // a run that was started and never waited for: its launch has ended by now
         pl->holds_fused = false;
         fused_turn_give();
@@ -1295,17 +1303,32 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->inst.swap(inst);
         return GDP_OK;
     }
-    GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), small_bytes, hipMemcpyHostToDevice, pl->stream));
+    // A flow plan (small): the tables go first, the kernel that prepares the cost buffers needs nothing else;
+    // the per-instance inputs follow on a second stream, beside that kernel.
+    size_t tables_bytes = small_bytes;
+    bool &split_upload = pl->split_upload;
+    {
+        std::lock_guard<std::mutex> lk(g_fused_mu);
+        split_upload = pl->flow_ready && !g_fused_busy;
+    }
+    if (split_upload) {
+        for (const auto &h : inst) tables_bytes = std::min(tables_bytes, h.off_inter);
+        split_upload = tables_bytes > 0 && tables_bytes < small_bytes;
+    }
+    GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), split_upload ? tables_bytes : small_bytes, hipMemcpyHostToDevice,
+                           pl->stream));
+    if (split_upload) {
+        // (the side stream is idle: whatever it last carried was joined to a main stream that has been waited for)
+        GDP_HIP(hipMemcpyAsync(pl->dbase + tables_bytes, stage.data() + tables_bytes, small_bytes - tables_bytes,
+                               hipMemcpyHostToDevice, pl->lane.side));
+        GDP_HIP(hipEventRecord(pl->lane.ev_side, pl->lane.side));
+    }
     {   // the parts of the cost buffers that no run ever overwrites
         const GdpDevInst *d_insts = reinterpret_cast<const GdpDevInst *>(pl->dbase + pl->off_insts);
         // A plan laid out for the flow launch gets NaN into its bands here if the turn is free right now (its
         // first run will most likely flow), else when a run first takes that way: a plan that finds the turn
         // taken every time never pays for it.
-        bool nan_bands = false;
-        if (pl->flow_ready) {
-            std::lock_guard<std::mutex> lk(g_fused_mu);
-            nan_bands = !g_fused_busy;
-        }
+        const bool nan_bands = split_upload;
         for (const Group &g : pl->groups) {
             if (!nan_bands)   // (one launch instead of three pays only where the three are short)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
@@ -1316,6 +1339,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                                            64 * GDP_VARIANTS[g.variant].r, nan_bands, g.sched.abort_flag, pl->stream));
         }
         pl->flow_clean = nan_bands;
+        if (split_upload) GDP_HIP(hipStreamWaitEvent(pl->stream, pl->lane.ev_side, 0));
     }
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
