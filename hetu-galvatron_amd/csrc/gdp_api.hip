@@ -885,10 +885,14 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // at work: the start of a task (four dependent round trips to memory before it reaches its gate) then
     // lies behind it when its cost rows appear.  So: the most waves per task that keep two layers' tasks
     // resident, else what keeps the most (ms per solve, 1 / 2 / 4 waves: S=22 V=16384 L=24 0.099 / 0.091 /
-    // 0.081; S=40 V=29493 L=28 - / 0.163 / 0.194).  With less than 0.4 of a layer resident the launch with
-    // completion counters and wide tiles is the faster one (flow against it, by resident share: S=22 V=65536
-    // L=24, 1.0: 0.17 against 0.23 ms; S=44 V=32768 L=32, 0.5: 0.43 against 0.55; S=40 V=60000 L=28, 0.44:
-    // 0.44 against 0.49; S=44 V=65536 L=32, 0.25: 0.84 against 0.42).  GALVATRON_DP_FLOW=1 asks for it
+    // 0.081; S=40 V=29493 L=28 - / 0.163 / 0.194).  It exists for the narrowest tile only, which is what a
+    // plan has when it is too small to fill the device with wider ones; for such plans it beat the launch
+    // with completion counters at every size measured (flow against it, by the share of a layer's tasks
+    // that is resident: S=22 V=65536 L=24, 1.0: 0.16 against 0.23 ms; S=44 V=32768 L=32, 0.5: 0.38 against
+    // 0.55; S=64 V=32768 L=16, 0.31: 0.31 against 0.35; S=88 V=16384 L=16, 0.27: 0.27 against 0.39; S=96
+    // V=16384 L=48, 0.25: 0.87 against 1.72).  Plans that get a wider tile run faster with the counters
+    // (forced onto the narrow tile and the flow launch: S=44 V=65536 L=32 0.63 against 0.64 ms, S=44
+    // V=131072 1.22 against 0.83, S=64 V=65536 L=16 0.62 against 0.45).  GALVATRON_DP_FLOW=1 asks for it
     // wherever the layout allows (costs only, no memory cost of 0, the tile of the latency variant).
     struct FlowPick { int K, nsrc; double resident; };
     auto flow_pick = [&](const Group &g) {
@@ -917,7 +921,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65534;
     for (const Group &g : pl->groups) {
         want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
-        if (want_flow && pl->flow_override != 1) want_flow = flow_pick(g).resident >= 0.4;
+        if (want_flow && pl->flow_override != 1) want_flow = flow_pick(g).resident >= 0.1;
     }
     pl->flow = pl->flow_ready = want_flow;
     if (want_flow) pl->fused = false;
