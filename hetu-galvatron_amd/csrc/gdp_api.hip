@@ -359,7 +359,6 @@ struct Group {  // instances with the same S, sorted by L descending
                                     // number of waves (1, 2, 4) that share the source strategies of a task
     int flow_nsrc = 0;              // flow launch: source strategies per wave (SU = flow_nsrc * latency)
     bool lat_ok = true;             // SU suits the latency variant of the per-layer kernel (a multiple of 8 * latency)
-    unsigned flow_lds = 0;          // flow launch: dynamic LDS that holds the workgroups per CU down (never touched)
     int flow_blocks = 0;            // flow launch: workgroups of the widest band (wave tasks incl. the parts of split ones)
     int chunk = 0;                  // instances taken through all their layers together; >= count: not chunked
     std::vector<int32_t> rows;      // chunked: {first instance, instances, layer} per grid row
@@ -1236,11 +1235,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             }
             g.slots = (int)((widest + 7) / 8 * g.xcd_group);
         }
-        if (const char *e = getenv("GALVATRON_DP_FLOW_WGS")) {
-            const int per_cu = atoi(e);
-            if (per_cu >= 1 && per_cu < 8 && pl->lds_per_cu >= 65536)
-                g.flow_lds = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
-        }
         sc->slots = g.slots;
         sc->spin_limit = pl->spin_limit;
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
@@ -1480,6 +1474,31 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
                     return bad("shape fields of a layer", k, l, 0);
                 if (y.lo < 0 || y.lo > h.ntile || y.hi < -1 || y.hi >= h.ntile || y.dep < 0) return bad("band of a layer", y.lo, y.hi, y.dep);
                 if ((long long)y.lo * tile_rows > h.ldm) return bad("filled rows beyond a row", k, l, y.lo);
+                if (y.fill_from < 0) return bad("first filled row of a layer", k, l, y.fill_from);   // (at or above the band: nothing to fill)
+                // What the band of this layer reads of the previous layer's output (rows u - mem[l-1][s'] for
+                // every row u of the band): in the pads, in the rows filled once per plan, or -- costs only --
+                // in the previous band.  A flow launch waits for every such cell, so each must get written;
+                // with the bands not closed (other launch schemes) the rows beyond the previous band belong
+                // to lanes whose results nobody reads.
+                if (l >= 1 && y.hi >= y.lo && !pl->keep_marks && !h.has_zero) {
+                    const GdpDevLayer &prev = lay[(size_t)k * g.max_L + (l - 1)];
+                    const gdp_problem *q = p[h.orig];
+                    long long mn = -1, mx = -1;
+                    for (int s2 = 0; s2 < h.S; ++s2) {
+                        const long long m = q->mem[(size_t)(l - 1) * h.S + s2];
+                        if (m >= h.V) continue;
+                        mn = mn < 0 ? m : std::min(mn, m);
+                        mx = std::max(mx, m);
+                    }
+                    if (mx >= 0) {
+                        const long long lowest = (long long)y.lo * tile_rows - mx;
+                        const long long highest = (long long)(y.hi + 1) * tile_rows - 1 - mn;
+                        if (lowest < -(long long)h.P) return bad("a band reads below the pad", k, l, lowest);
+                        if (lowest >= 0 && lowest < prev.fill_from) return bad("a band reads below the filled rows", k, l, lowest);
+                        const long long written_to = prev.hi >= prev.lo ? (long long)(prev.hi + 1) * tile_rows : (long long)prev.lo * tile_rows;
+                        if (pl->flow_ready && highest >= written_to) return bad("a band of a flow plan reads above the previous band", k, l, highest);
+                    }
+                }
             }
         }
         for (size_t r = 0; r + 2 < g.rows.size(); r += 3) {
@@ -1494,6 +1513,15 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
             const long long grid_x = 8LL * (g.rows.empty() ? g.active[(size_t)seg.first] : g.chunk) * g.slots;
             if (grid_x < 1 || grid_x > 0x7fffffffLL || g.slots < 1) return bad("grid of a fused launch", grid_x, g.slots, 0);
             if (seg.lds_bytes > 65536u) return bad("dynamic LDS of a fused launch", seg.lds_bytes, 0, 0);
+        }
+        if (pl->flow_ready) {
+            // flow launch: grid = (workgroups of the widest band, layers, instances); a task's row offsets are
+            // ro[part * nsrc + u], u < nsrc (inside the SU entries checked below), its cost rows and gate cells
+            // the elements a per-layer task reads
+            if (g.flow_blocks < 0 || g.max_L > 65535 || g.count > 65535) return bad("grid of a flow launch", g.flow_blocks, g.max_L, g.count);
+            bool known = false;
+            for (int c : GDP_FLOW_NSRC) known = known || c == g.flow_nsrc;
+            if (!known || 2 * g.flow_nsrc > 64) return bad("sources per wave of a flow task", g.flow_nsrc, 0, 0);
         }
         const long long tasks = (long long)g.max_ntile * g.ntb * (g.latency > 1 ? g.latency : 1);
         if (tasks / GDP_WAVES_PER_BLOCK + 16 > 0x7fffffffLL || g.count > 65535) return bad("grid of a per-layer launch", tasks, g.count, 0);
@@ -1579,7 +1607,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
             if (g.flow_blocks > 0)
                 GDP_HIP(gdp_launch_relax_flow(g.flow_nsrc, g.latency, g.sched.lay, g.max_L, g.count, g.flow_blocks, g.SP, 0, g.max_L,
-                                              g.sched.abort_flag, pl->spin_limit, g.flow_lds, pl->stream));
+                                              g.sched.abort_flag, pl->spin_limit, pl->stream));
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
             ++li;
         }

@@ -162,8 +162,7 @@ static const int GDP_FLOW_NSRC[] = {8, 12, 16, 20, 24};
 // The cells the launch writes must hold NaN beforehand and the abort flag zero: gdp_launch_flow_reset
 // (bands of all layers of n_inst instances).
 hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
-                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, unsigned lds_bytes,
-                                 hipStream_t stream);
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, hipStream_t stream);
 hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
                                  int max_L, int tile_rows, int32_t *abort_flag, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);

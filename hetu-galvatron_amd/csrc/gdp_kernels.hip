@@ -1426,15 +1426,14 @@ hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched
 }
 
 hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
-                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, unsigned lds_bytes,
-                                 hipStream_t stream)
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, hipStream_t stream)
 {
     if (n_inst < 1 || n_inst > 65535 || layers < 1 || layers > 65535 || grid_blocks < 1) return hipErrorInvalidValue;
     const unsigned ntb = (unsigned)(SP / GDP_LAT_TS) * (unsigned)latency;  // with the parts of a split task
     dim3 grid((unsigned)grid_blocks, (unsigned)layers, (unsigned)n_inst), block(64 * GDP_WAVES_PER_BLOCK);
 #define X(NSRC, K)                                                                                                   \
     if (nsrc == NSRC && latency == K) {                                                                              \
-        hipLaunchKernelGGL((gdp_relax_flow_kernel<NSRC, K>), grid, block, lds_bytes, stream, lay, max_L, layer0, ntb, \
+        hipLaunchKernelGGL((gdp_relax_flow_kernel<NSRC, K>), grid, block, 0, stream, lay, max_L, layer0, ntb, \
                            abort_flag, spin_limit);                                                                  \
         return hipGetLastError();                                                                                    \
     }

@@ -194,3 +194,36 @@ def test_flow_plans_from_several_threads(golden):
         t.join()
     assert not errors, errors
     assert any(flowed)
+
+
+def test_flow_alternating_problems_in_the_same_memory():
+    """Two different problems of one shape solved in turn: the library hands the second the device
+    memory the first has just left (same layout, same addresses), so a cost cell or cache line that
+    survived from the other problem's run would show up as a wrong result."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    rng = np.random.Generator(np.random.PCG64(77))
+    L, S, V = 12, 22, 6000
+    a = W.random_instance(rng, L, S, V, mem_hi=300, inf_frac=0.05, n_keys=3)
+    # same memory costs (same bands, same layout), other times: every cell differs
+    b = W.Instance("b", a.mem.copy(), a.intra * 1.7 + 0.25, a.inter * 0.6, a.V, dict(a.other_mem), dict(a.other_time),
+                   None if a.inter_tables is None else a.inter_tables * 0.6, a.inter_index)
+    want = {}
+    for name, inst in (("a", a), ("b", b)):
+        wt, wr, wm, _, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+        want[name] = (wt, wr, wm)
+    assert want["a"][0] != want["b"][0]
+    keys = sorted(a.other_mem)
+    for it in range(40):
+        name, inst = (("a", a), ("b", b))[it % 2]
+        prob = _problem(inst)
+        if it % 8 < 6:
+            _lib.solve_batch([prob])
+        else:
+            with _lib.Plan([prob]) as plan:
+                for _ in range(2):
+                    t = plan.run(1)
+                    assert t.flow == 1
+                    plan.fetch()
+        H.assert_same_results(_results(prob, keys), want[name], f"iteration {it} problem {name}")
