@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the layer-wise DP hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg0|cfg1|cfg4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg0|cfg1|cfg4|galvatron_like]
 
 One "step" is one complete solve of the workload on the device: every layer's relaxation kernel
 over every instance of the batch, plus the on-device backtrack, with the inputs already resident
@@ -38,6 +38,8 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    the backtrack recomputes the argmin of the L cells on its path.  ``with_mark_table``
                    reports the mode that stores the reference's argmin table instead: 17 bytes and
                    five instead of two vector instructions per relaxation).
+* ``config.plugin_call_ms``  one call of the drop-in ``galvatron_dp_core.dynamic_programming_core`` with the
+                   reference's eleven arguments (single instances; median of a few calls).
 * ``config.search_wall_ms_from_host_arrays``  the same solve through gdp_solve_batch from host arrays
                    (validation, layout, upload, all kernels, download; median of a few calls), beside
                    ``search_wall_ms_device`` (first kernel to last kernel of one solve, HIP events).
@@ -128,6 +130,8 @@ def _problems(workload: str, compute_all: bool = True, keep_marks: bool = False)
     from galvatron_dp import _lib, workloads as W
     if workload == "cfg3":
         insts = W.config3()
+    elif workload == "galvatron_like":
+        insts = [W.galvatron_like()]      # the shape of one DPAlg.fit call of a real search (L=28, S=40, V=29493)
     else:
         insts = [W.CONFIGS[int(workload[3:])]()]
     probs = []
@@ -145,7 +149,8 @@ def _cpu_baseline(workload: str, budget_s: float = 15.0):
     import numpy as np
     from galvatron_dp import workloads as W
     from oracle import dp_oracle as O
-    inst = W.config3(n_limit=1)[0] if workload == "cfg3" else W.CONFIGS[int(workload[3:])]()
+    inst = (W.config3(n_limit=1)[0] if workload == "cfg3" else W.galvatron_like() if workload == "galvatron_like"
+            else W.CONFIGS[int(workload[3:])]())
     use_ref = O.ref_available()
     fn = O.ref_solve if use_ref else O.solve
     per_layer = inst.V * inst.S * inst.S
@@ -203,7 +208,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "galvatron_like"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--row-skipping", action="store_true",
                     help="time the library's default (rows that need no arithmetic are filled or left out) instead "
@@ -214,7 +219,7 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true",
                     help="leave out the row-skipping and mark-table legs (profiling runs: the trace then holds the "
                          "headline's launches alone)")
-    ap.add_argument("--also", default="cfg3,cfg0,cfg1,cfg4", help="comma-separated extra workloads summarised in the same line")
+    ap.add_argument("--also", default="cfg3,cfg0,cfg1,cfg4,galvatron_like", help="comma-separated extra workloads summarised in the same line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run three device-to-device copies of 1 GiB (a kernel of known traffic, to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
@@ -278,6 +283,22 @@ def main() -> int:
             _lib.solve_batch(probs)
             host_ms.append((time.perf_counter() - h0) * 1e3)
         host_ms = sorted(host_ms[1:])[len(host_ms[1:]) // 2] if host_leg else None
+        # ... and as ONE call of the drop-in plugin with the reference's eleven arguments (the caller's arrays
+        # allocated once, as DPAlg does), for single instances.
+        plugin_ms = None
+        if host_leg and len(insts) == 1:
+            import numpy as np
+            import galvatron_dp_core as plugin
+            i0 = insts[0]
+            res = {k: np.full(i0.L, -1, dtype=np.int32) for k in i0.other_mem}
+            inter = np.ascontiguousarray(i0.inter)
+            args = (i0.L, i0.V, i0.S, i0.mem, None, None, inter, i0.intra, i0.other_mem, i0.other_time, res)
+            times = []
+            for _ in range(1 + max(5, min(steps, 30))):
+                h0 = time.perf_counter()
+                plugin.dynamic_programming_core(*args)
+                times.append((time.perf_counter() - h0) * 1e3)
+            plugin_ms = sorted(times[1:])[len(times[1:]) // 2]
         relax = tm.relaxations
         launches = tm.relax_launches
         avg_launch_s = tm.relax_ms * 1e-3 / launches
@@ -290,7 +311,7 @@ def main() -> int:
         return {
             "insts": insts, "probs": probs, "relaxations": relax, "ms_per_step": wall / steps * 1e3,
             "value": relax * steps / wall, "launches": launches, "avg_launch_ms": avg_launch_s * 1e3,
-            "device_ms": t1.total_ms, "host_ms": host_ms, "executed_fraction": tm.executed / relax,
+            "device_ms": t1.total_ms, "host_ms": host_ms, "plugin_ms": plugin_ms, "executed_fraction": tm.executed / relax,
             "tops_issued": issued * per_launch_s / 1e12, "tops_reference": 3.0 * per_launch_s / 1e12,
             "issued_per_relaxation": issued,
             "gbs": tm.relax_bytes / launches / avg_launch_s / 1e9,
@@ -327,7 +348,8 @@ def main() -> int:
                    "argmin": ("stored while relaxing (one byte per cell)" if a.mark_table else
                               "recomputed on the backtrack (costs-only relaxation)"),
                    "search_wall_ms_device": m["device_ms"],
-                   "search_wall_ms_from_host_arrays": m["host_ms"], "launch_scheme": m["scheme"],
+                   "search_wall_ms_from_host_arrays": m["host_ms"], "plugin_call_ms": m["plugin_ms"],
+                   "launch_scheme": m["scheme"],
                    "register_tile": m["tile"],
                    "relaxations_executed_fraction": m["executed_fraction"], "bit_exact": m["bit_exact"],
                    "device": _lib.device_info()},
@@ -348,7 +370,8 @@ def main() -> int:
         mm = measure(w, max(3, a.steps // 4), 1, host_leg=not a.headline_only, check=True)
         ff = fractions(mm)
         also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
-                   "search_wall_ms_from_host_arrays": mm["host_ms"],
+                   "search_wall_ms_device": mm["device_ms"],
+                   "search_wall_ms_from_host_arrays": mm["host_ms"], "plugin_call_ms": mm["plugin_ms"],
                    "launch_scheme": mm["scheme"], "kernel": mm["kernel"], "register_tile": mm["tile"],
                    "roofline_frac_valu_fp64": ff["frac"], "issued_ops_per_relaxation": mm["issued_per_relaxation"],
                    "roofline_frac_valu_fp64_reference_ops": ff["frac_reference_ops"],

@@ -169,6 +169,26 @@ def config4(seed: int = DEFAULT_SEED + 4, random_other_time: bool = False,
     return Instance("cfg4", mem, intra, _shared(tables, index), V, om, ot, tables, index)
 
 
+def galvatron_like() -> Instance:
+    """Shape of a real search-engine call: 28 identical layers, inter made of zeros and
+    the 1e-10..3e-9 ordering sentinels, first layer's inter zeroed, four keys
+    (dynamic_programming.py:241,266,347-372).  Numbers are synthetic."""
+    rng = np.random.Generator(np.random.PCG64(77))
+    L, S, V = 28, 40, 29493
+    mem_row = rng.integers(300, 2600, size=S)
+    t_row = np.round(rng.uniform(20, 60, size=S), 3)
+    m = np.zeros((S, S))
+    sent = np.array([0.0, 1e-10, 1e-9, 2e-9, 3e-9, 0.37, 1.21])
+    m[:] = sent[rng.integers(0, len(sent), size=(S, S))]
+    np.fill_diagonal(m, 0.0)
+    inter = np.repeat(m[None], L, 0)
+    inter[0] = 0.0
+    om = {1: 4100, 2: 2300, 4: 1500, 8: 900}
+    ot = {1: 31.5, 2: 17.25, 4: 9.125, 8: 6.0625}
+    return Instance("galvatron_like", np.repeat(mem_row[None], L, 0).astype(np.int32),
+                      np.repeat(t_row[None], L, 0), inter, V, om, ot, inter, np.arange(L, dtype=np.int32))
+
+
 CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4}
 
 

@@ -96,28 +96,8 @@ def build_case(builder: str, kw: dict) -> W.Instance:
             inst.mem[big] = rng.integers(1, max(2, kw["V"] // (kw["L"] + 1)), size=int(big.sum()))
         return inst
     if builder == "galvatron_like":
-        return galvatron_like()
+        return W.galvatron_like()
     return getattr(W, builder)(**kw)
-
-
-def galvatron_like() -> W.Instance:
-    """Shape of a real search-engine call: 28 identical layers, inter made of zeros and
-    the 1e-10..3e-9 ordering sentinels, first layer's inter zeroed, four keys
-    (dynamic_programming.py:241,266,347-372).  Numbers are synthetic."""
-    rng = np.random.Generator(np.random.PCG64(77))
-    L, S, V = 28, 40, 29493
-    mem_row = rng.integers(300, 2600, size=S)
-    t_row = np.round(rng.uniform(20, 60, size=S), 3)
-    m = np.zeros((S, S))
-    sent = np.array([0.0, 1e-10, 1e-9, 2e-9, 3e-9, 0.37, 1.21])
-    m[:] = sent[rng.integers(0, len(sent), size=(S, S))]
-    np.fill_diagonal(m, 0.0)
-    inter = np.repeat(m[None], L, 0)
-    inter[0] = 0.0
-    om = {1: 4100, 2: 2300, 4: 1500, 8: 900}
-    ot = {1: 31.5, 2: 17.25, 4: 9.125, 8: 6.0625}
-    return W.Instance("galvatron_like", np.repeat(mem_row[None], L, 0).astype(np.int32),
-                      np.repeat(t_row[None], L, 0), inter, V, om, ot, inter, np.arange(L, dtype=np.int32))
 
 
 def solve_case(item):
