@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define GDP_VERSION 100 /* major*10000 + minor*100 + patch */
+#define GDP_VERSION 101 /* major*10000 + minor*100 + patch */
 
 /* return codes */
 #define GDP_OK 0

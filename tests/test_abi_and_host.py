@@ -27,7 +27,7 @@ def test_header_symbols_are_exported():
 
 
 def test_version_and_struct_sizes():
-    assert _lib.lib().gdp_version() == 100
+    assert _lib.lib().gdp_version() == 101
     assert ctypes.sizeof(_lib.gdp_problem) == 80
     assert ctypes.sizeof(_lib.gdp_result) == 40
     assert ctypes.sizeof(_lib.gdp_timing) == 64
