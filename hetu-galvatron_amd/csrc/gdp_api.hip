@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -313,6 +314,26 @@ void fused_turn_take()
 // The turn if it is free.  A flow plan that finds it taken does not queue up for it: it runs that solve
 // with one launch per layer, beside the launch that holds the turn (threads that call the plugin side by
 // side, as the reference's parallel search does, then overlap instead of taking turns).
+// When a launch whose workgroups wait was given up although nobody had shortened its waits, something else
+// holds places on the device -- most likely another process with such launches of its own (the turn above
+// orders the threads of this process only).  Every further launch of that kind would risk the same
+// wait of a good part of a second, so for the next while the library chooses launches that never wait
+// (one per layer) where the choice is its own; a caller's explicit request still counts.
+constexpr int64_t DEFAULT_SPIN_LIMIT = 1 << 18;
+constexpr double SHARED_DEVICE_BACKOFF_S = 30.0;
+std::atomic<int64_t> g_last_give_up_ms{-1};   // steady clock, milliseconds; -1: never
+
+int64_t steady_ms()
+{
+    return std::chrono::duration_cast<std::chrono::milliseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+bool device_seems_shared()
+{
+    const int64_t t = g_last_give_up_ms.load(std::memory_order_relaxed);
+    return t >= 0 && (double)(steady_ms() - t) < SHARED_DEVICE_BACKOFF_S * 1e3;
+}
+
 bool fused_turn_try_take()
 {
     std::lock_guard<std::mutex> lk(g_fused_mu);
@@ -468,7 +489,7 @@ struct gdp_plan {
     int flow_override = -1;       // GALVATRON_DP_FLOW=0|1: never / wherever the layout allows
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
-    int64_t spin_limit = 1 << 18; // polls a waiting wave makes before the launch is abandoned: about a second
+    int64_t spin_limit = DEFAULT_SPIN_LIMIT; // polls a waiting wave makes before the launch is abandoned: about a second
                                   // (3.5 us apart), a thousand times the longest wait of a healthy launch
     size_t off_zero = 0, zero_words = 0, off_abort = 0;
     int num_cu = 0;
@@ -870,7 +891,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             }
         }
         band_frac = all > 0 ? live / all : 1.0;
-        if (!fused_preset) pl->fused = first_layer * band_frac >= 2.0 * pl->num_cu;
+        if (!fused_preset) pl->fused = first_layer * band_frac >= 2.0 * pl->num_cu && !device_seems_shared();
     }
     // Launches that small run one or two waves per SIMD, and what they wait for is memory latency, not
     // instruction issue: their narrowest tile has a variant built for that (measured, 16 layers, one
@@ -916,7 +937,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         }
         return best;
     };
-    bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused) : !fused_preset;
+    bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused)
+                                            : !fused_preset && !device_seems_shared();
     want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65534;
     for (const Group &g : pl->groups) {
         want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
@@ -1668,6 +1690,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
         pl->fused = false;
         pl->flow = false;
         pl->fused_gave_up = true;
+        if (pl->spin_limit >= DEFAULT_SPIN_LIMIT) g_last_give_up_ms.store(steady_ms(), std::memory_order_relaxed);
         if (pl->no_fallback)
             return fail(GDP_E_HIP, "fused launch: a bounded wait ran out before its tiles were finished");
         return run(pl, mode, t);
@@ -1884,6 +1907,11 @@ int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_c
         if (!marks_possible) break;
     }
     return GDP_OK;
+}
+
+void gdp_debug_shared_device(int32_t seems_shared)
+{
+    g_last_give_up_ms.store(seems_shared ? steady_ms() : -1, std::memory_order_relaxed);
 }
 
 void gdp_cache_trim(void)

@@ -39,7 +39,7 @@ GDP_STATIC_SCRATCH_BYTES = 64 << 20
 
 EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_solve_static", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
                     "gdp_plan_destroy", "gdp_plan_set_option", "gdp_cache_trim", "gdp_last_error", "gdp_version",
-                    "gdp_device_info", "gdp_debug_check_layout")
+                    "gdp_device_info", "gdp_debug_check_layout", "gdp_debug_shared_device")
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -114,6 +114,8 @@ def lib() -> ctypes.CDLL:
         L.gdp_device_info.restype = ctypes.c_int
         L.gdp_debug_check_layout.argtypes = [ctypes.c_int32, pp, ctypes.c_int32, ctypes.c_int64]
         L.gdp_debug_check_layout.restype = ctypes.c_int
+        L.gdp_debug_shared_device.argtypes = [ctypes.c_int32]
+        L.gdp_debug_shared_device.restype = None
         _lib = L
     return _lib
 
@@ -219,6 +221,12 @@ def check_layout(problems: Sequence[Problem], num_cu: int = 256, lds_per_cu: int
     every address the kernels would form; raises with the violated bound."""
     P, _ = _arrays(problems)
     _check(lib().gdp_debug_check_layout(len(problems), P, num_cu, lds_per_cu))
+
+
+def debug_shared_device(seems_shared: bool) -> None:
+    """gdp_debug_shared_device: puts the library into (or takes it out of) the state it enters when a waiting
+    launch was given up: launches that never wait are then chosen wherever the choice is the library's."""
+    lib().gdp_debug_shared_device(1 if seems_shared else 0)
 
 
 def solve_static(problem: Problem) -> None:

@@ -194,6 +194,13 @@ void gdp_cache_trim(void);
  * environment (GALVATRON_DP_FUSED, _SKIP, _TILE_TS, _TILE_R, _CHUNK, _LATENCY_VARIANT ...) apply. */
 int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_cu, int64_t lds_per_cu);
 
+/* Test aid (no counterpart in the reference).  After a launch whose workgroups wait (GDP_OPT_FUSED,
+ * GDP_OPT_FLOW) has been given up with the default spin limit, the library takes the device to be shared
+ * with another process and, for the next 30 seconds, chooses one launch per layer wherever the choice is
+ * its own (explicit requests -- flags, options, environment -- still count).  This call puts the library
+ * into that state (1) or ends it (0) without a launch having to time out. */
+void gdp_debug_shared_device(int32_t seems_shared);
+
 /* Text of the calling thread's last error ("" if none). */
 const char *gdp_last_error(void);
 /* GDP_VERSION of the built library. */

@@ -227,3 +227,36 @@ def test_flow_alternating_problems_in_the_same_memory():
                     assert t.flow == 1
                     plan.fetch()
         H.assert_same_results(_results(prob, keys), want[name], f"iteration {it} problem {name}")
+
+
+def test_launches_that_never_wait_on_a_device_that_seems_shared(golden):
+    """After a waiting launch was given up with the default spin limit the library takes the device to
+    be shared and chooses one launch per layer where the choice is its own; an explicit request still
+    counts; the state ends by itself (here: is ended by the test aid)."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    rec = golden["cfg0"]
+    inst = H.build_case(rec)
+    big = golden["cfg2_small"]
+    big_inst = H.build_case(big)
+    try:
+        _lib.debug_shared_device(True)
+        for r, i in ((rec, inst), (big, big_inst)):
+            prob = _problem(i)
+            with _lib.Plan([prob]) as plan:
+                t = plan.run(1)
+                plan.fetch()
+                assert t.flow == 0 and t.fused == 0 and t.relax_launches == i.L
+                _check_against_golden(prob, r, "seems shared")
+        prob = _problem(big_inst, launch="fused")
+        with _lib.Plan([prob]) as plan:
+            assert plan.run(1).fused == 1
+            plan.fetch()
+            _check_against_golden(prob, big, "explicit request")
+    finally:
+        _lib.debug_shared_device(False)
+    prob = _problem(inst)
+    with _lib.Plan([prob]) as plan:
+        assert plan.run(1).flow == 1
+        plan.fetch()
+        _check_against_golden(prob, rec, "afterwards")
