@@ -916,7 +916,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // wherever the layout allows (costs only, no memory cost of 0, the tile of the latency variant).
     struct FlowPick { int K, nsrc; double resident; };
     auto flow_pick = [&](const Group &g) {
-        auto waves_per_simd = [](int nsrc) { return nsrc <= 8 ? 7 : nsrc <= 12 ? 6 : nsrc <= 16 ? 5 : nsrc <= 20 ? 4 : 3; };  // by their registers
+        auto waves_per_simd = [](int nsrc) { return nsrc <= 12 ? 8 : nsrc <= 16 ? 7 : nsrc <= 20 ? 6 : 5; };  // by their registers (38 + 2 per source)
         auto nsrc_for = [&](int K) {
             for (int c : GDP_FLOW_NSRC)
                 if (c * K >= g.S) return c;
