@@ -900,7 +900,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // Small and middling plans run all their layers in one launch that waits on the cost cells themselves
     // (gdp_relax_flow_kernel) -- unless the caller asked for a launch scheme: per-layer launches are also
     // what a shared device wants, since they never wait.  A flow task asks for all its cost rows at once,
-    // at most 24 per wave (they wait in registers), so its sources go on 1, 2 or 4 waves.  More waves
+    // at most 32 per wave (they wait in registers), so its sources go on 1, 2 or 4 waves.  More waves
     // shorten the task -- as long as the next layers' tasks still find room on the device beside the layer
     // at work: the start of a task (four dependent round trips to memory before it reaches its gate) then
     // lies behind it when its cost rows appear.  So: the most waves per task that keep two layers' tasks
@@ -916,7 +916,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // wherever the layout allows (costs only, no memory cost of 0, the tile of the latency variant).
     struct FlowPick { int K, nsrc; double resident; };
     auto flow_pick = [&](const Group &g) {
-        auto waves_per_simd = [](int nsrc) { return nsrc <= 12 ? 8 : nsrc <= 16 ? 7 : nsrc <= 20 ? 6 : 5; };  // by their registers (38 + 2 per source)
+        auto waves_per_simd = [](int nsrc) { return nsrc <= 12 ? 8 : nsrc <= 16 ? 7 : nsrc <= 20 ? 6 : nsrc <= 28 ? 5 : 4; };  // by their registers (38 + 2 per source)
         auto nsrc_for = [&](int K) {
             for (int c : GDP_FLOW_NSRC)
                 if (c * K >= g.S) return c;
@@ -941,7 +941,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                                             : !fused_preset && !device_seems_shared();
     want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65534;
     for (const Group &g : pl->groups) {
-        want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= 4 * 24;
+        want_flow = want_flow && g.latency_possible(pl->keep_marks) && g.count <= 65535 && g.S <= GDP_FLOW_MAX_S;
         if (want_flow && pl->flow_override != 1) want_flow = flow_pick(g).resident >= 0.1;
     }
     pl->flow = pl->flow_ready = want_flow;

@@ -153,8 +153,10 @@ hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched
                                   int layers, unsigned lds_bytes, hipStream_t stream);
 // (sources per wave, waves per task) of the flow kernels that are built
 #define GDP_FOR_EACH_FLOW(X) \
-    X(8, 1) X(12, 1) X(16, 1) X(20, 1) X(24, 1) X(8, 2) X(12, 2) X(16, 2) X(20, 2) X(24, 2) X(8, 4) X(12, 4) X(16, 4) X(20, 4) X(24, 4)
-static const int GDP_FLOW_NSRC[] = {8, 12, 16, 20, 24};
+    X(8, 1) X(12, 1) X(16, 1) X(20, 1) X(24, 1) X(28, 1) X(32, 1) X(8, 2) X(12, 2) X(16, 2) X(20, 2) X(24, 2) X(28, 2) X(32, 2) \
+    X(8, 4) X(12, 4) X(16, 4) X(20, 4) X(24, 4) X(28, 4) X(32, 4)
+static const int GDP_FLOW_NSRC[] = {8, 12, 16, 20, 24, 28, 32};
+#define GDP_FLOW_MAX_S (4 * 32)   // most sources per wave x most waves per task
 // Layers layer0 .. layer0+layers-1 of the first n_inst instances of a group in one launch whose tasks
 // wait on the cost cells themselves (gdp_relax_flow_kernel; costs only, the tile of the latency variant,
 // `latency` = waves that share the sources of a task, nsrc = sources per wave: one of GDP_FLOW_NSRC, the

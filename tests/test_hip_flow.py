@@ -34,7 +34,7 @@ def _check_against_golden(prob, rec, name):
     H.assert_same_results(got, H.golden_results(rec), name)
 
 
-@pytest.mark.parametrize("S", [1, 7, 8, 9, 12, 13, 22, 24, 25, 40, 44, 48, 49, 63, 96])
+@pytest.mark.parametrize("S", [1, 7, 8, 9, 12, 13, 22, 24, 25, 29, 33, 40, 44, 48, 49, 63, 65, 96, 97, 128])
 def test_flow_launch_matches_the_oracle(S, monkeypatch):
     """Small instances run as one flow launch by default; sources on 1, 2 and 4 waves per task where S
     allows (S on both sides of every sources-per-wave step); f of the last layer compared too, and the
@@ -64,7 +64,7 @@ def test_flow_launch_matches_the_oracle(S, monkeypatch):
                         assert prob.f_out.tobytes() == wf.tobytes()
             seen.append(t.latency_variant)
     for preset, k in zip(("1", "2", "4"), seen[2::2]):
-        if S <= 24 * int(preset):
+        if S <= 32 * int(preset):
             assert k == int(preset), (preset, seen)
 
 
