@@ -378,6 +378,7 @@ struct Group {  // instances with the same S, sorted by L descending
     int max_V = 0;
     int latency = 0;                // per-layer launches use the variant for launches with few waves: 0, or the
                                     // number of waves (1, 2, 4) that share the source strategies of a task
+    bool any_fill = false;          // some layer of some instance has rows below its band that are filled once per plan
     int flow_nsrc = 0;              // flow launch: source strategies per wave (SU = flow_nsrc * latency)
     bool lat_ok = true;             // SU suits the latency variant of the per-layer kernel (a multiple of 8 * latency)
     int flow_blocks = 0;            // flow launch: workgroups of the widest band (wave tasks incl. the parts of split ones)
@@ -1224,6 +1225,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                     y.fill_from = (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
                 }
                 y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
+                if ((int64_t)h_band[(size_t)(g.first + k)][3 * (size_t)l + 1] * (64 * GDP_VARIANTS[h.variant].r) > y.fill_from)
+                    g.any_fill = true;
                 y.lo = h_band[(size_t)(g.first + k)][3 * (size_t)l + 1];
                 y.hi = h_band[(size_t)(g.first + k)][3 * (size_t)l + 2];
                 if (y.hi >= y.lo)
@@ -1353,7 +1356,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             if (!nan_bands)   // (one launch instead of three pays only where the three are short)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                         64 * GDP_VARIANTS[g.variant].r,
-                                        GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks ? 0 : GDP_INIT_FILL), pl->stream));
+                                        GDP_INIT_PADS | GDP_INIT_ZERO | (pl->keep_marks || !g.any_fill ? 0 : GDP_INIT_FILL),
+                                        pl->stream));
             else
                 GDP_HIP(gdp_launch_prepare(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                            64 * GDP_VARIANTS[g.variant].r, nan_bands, g.sched.abort_flag, pl->stream));
@@ -1603,7 +1607,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
         if (what)
             for (const Group &g : pl->groups)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
-                                        64 * GDP_VARIANTS[g.variant].r, what, pl->stream));
+                                        64 * GDP_VARIANTS[g.variant].r, g.any_fill ? what : (what & ~GDP_INIT_FILL), pl->stream));
     }
     size_t li = 0;
 
