@@ -260,3 +260,32 @@ def test_launches_that_never_wait_on_a_device_that_seems_shared(golden):
         assert plan.run(1).flow == 1
         plan.fetch()
         _check_against_golden(prob, rec, "afterwards")
+
+
+def test_flow_launch_on_the_fuzz_shapes_without_exports():
+    """The shapes of the differential test (V from 1 to 4099, S around every tile and wave width), run as
+    callers run them: nothing exported, so only the bands are computed (closed under reading) and rows
+    below them are filled where something reads them.  Results against the oracle; memory costs small,
+    large, beyond the budget; +inf costs; ties."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    from test_hip_fuzz import SHAPES
+    flowed = 0
+    for n, (L, S, V) in enumerate(SHAPES):
+        for variant in range(4):
+            rng = np.random.Generator(np.random.PCG64([91, n, variant]))
+            hi = [max(1, V // (L + 1)), max(1, V // 2), V + 3, 3][variant]
+            inst = W.random_instance(rng, L, S, V, integer_costs=variant in (1, 3), mem_hi=hi,
+                                     per_layer_inter=bool(variant % 2), inf_frac=0.2 if variant >= 2 else 0.0,
+                                     over_frac=0.1 if variant == 3 else 0.0, n_keys=min(4, 1 + variant))
+            wt, wr, wm, _, _ = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+            keys = sorted(inst.other_mem)
+            prob = _problem(inst)
+            with _lib.Plan([prob]) as plan:
+                for rep in range(2):
+                    t = plan.run(1)
+                    plan.fetch()
+                    flowed += t.flow
+                    H.assert_same_results(_results(prob, keys), (wt, wr, wm), f"shape {(L, S, V)} variant {variant} run {rep}")
+    assert flowed > len(SHAPES)
