@@ -362,7 +362,41 @@ struct HostInst {
     size_t off_H, off_M, off_inter, off_intra, off_index, off_roff, off_mem;
     bool has_zero = false;  // some memory cost is 0 (see gdp_launch_zero_pass)
     size_t off_zcols = 0;
+    // a dense [L,S,S] transition array whose equal matrices are kept once (share_equal_matrices):
+    std::vector<int32_t> mat_of;   // layer -> kept matrix
+    std::vector<int32_t> mat_src;  // kept matrix -> the layer whose copy is taken
+    int matrix(const gdp_problem *q, int l) const { return q->inter_index ? q->inter_index[l] : mat_of[(size_t)l]; }
 };
+
+// The reference's callers pass one transition matrix per layer, and almost all of them are copies of a
+// few (galvatron/core/search_engine/dynamic_programming.py:368-372: one matrix per layer type, repeated
+// for its layers, the first layer's zeroed).  Matrices with the same bytes are kept once: the layers in
+// flight then share their transition costs in the caches instead of each fetching its own copy
+// (measured per call from host arrays, 32 equal matrices of 44 x 44: 0.81 -> 0.60 ms; 48 of 88 x 88:
+// 6.65 -> 6.26 ms), and the upload shrinks.  A layer is compared with the matrix of the layer before it
+// and, failing that, with the first few kept ones; comparisons of different matrices end at the first
+// byte that differs, so an array of L different matrices costs next to nothing to look through.
+void share_equal_matrices(const gdp_problem *q, HostInst &h)
+{
+    constexpr size_t LOOKED_AT = 8;
+    const size_t bytes = sizeof(double) * (size_t)q->S * q->S;
+    auto mat = [&](int l) { return reinterpret_cast<const char *>(q->inter) + (size_t)l * bytes; };
+    h.mat_of.assign((size_t)q->L, 0);
+    h.mat_src.clear();
+    for (int l = 0; l < q->L; ++l) {
+        int found = -1;
+        const int before = l > 0 ? h.mat_of[(size_t)l - 1] : -1;
+        if (before >= 0 && memcmp(mat(l), mat(h.mat_src[(size_t)before]), bytes) == 0) found = before;
+        for (size_t t = 0; found < 0 && t < std::min(h.mat_src.size(), LOOKED_AT); ++t)
+            if ((int)t != before && memcmp(mat(l), mat(h.mat_src[t]), bytes) == 0) found = (int)t;
+        if (found < 0) {
+            found = (int)h.mat_src.size();
+            h.mat_src.push_back(l);
+        }
+        h.mat_of[(size_t)l] = found;
+    }
+    h.n_inter = (int)h.mat_src.size();
+}
 
 struct Group {  // instances with the same S, sorted by L descending
     int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt;
@@ -569,7 +603,7 @@ int gdp_validate(const gdp_problem *p, int i)
         *m_out = m;
         return true;
     };
-    constexpr int TMAX_KEPT = 64;
+    constexpr int TMAX_KEPT = 1024;   // 8 KB of stack
     double tmax[TMAX_KEPT];
     const bool kept = p->inter_index && T <= TMAX_KEPT;
     if (p->inter_index)  // every matrix is checked, also one that no layer uses
@@ -767,6 +801,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.SU = (int)align_up((size_t)q->S, GDP_SRC_UNROLL);
         h.n_key = q->n_key;
         h.n_inter = q->inter_index ? q->n_inter : q->L;
+        if (!q->inter_index) share_equal_matrices(q, h);
         h.flags = q->flags;
         int maxm = 0;
         for (size_t k = 0; k < (size_t)q->L * q->S; ++k) {
@@ -1124,15 +1159,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
         // inter: [T][rows][SP], zero padded
         double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
-        for (int t = 0; t < h.n_inter; ++t)
+        for (int t = 0; t < h.n_inter; ++t) {
+            const double *from = q->inter + (size_t)(q->inter_index ? t : h.mat_src[(size_t)t]) * h.S * h.S;
             for (int a = 0; a < h.S; ++a)
-                memcpy(it + ((size_t)t * rows + a) * h.SP, q->inter + ((size_t)t * h.S + a) * h.S,
-                       sizeof(double) * (size_t)h.S);
+                memcpy(it + ((size_t)t * rows + a) * h.SP, from + (size_t)a * h.S, sizeof(double) * (size_t)h.S);
+        }
         double *ia = reinterpret_cast<double *>(stage.data() + h.off_intra);
         for (int l = 0; l < h.L; ++l)
             memcpy(ia + (size_t)l * h.SP, q->intra + (size_t)l * h.S, sizeof(double) * (size_t)h.S);
         int32_t *ix = reinterpret_cast<int32_t *>(stage.data() + h.off_index);
-        for (int l = 0; l < h.L; ++l) ix[l] = q->inter_index ? q->inter_index[l] : l;
+        for (int l = 0; l < h.L; ++l) ix[l] = h.matrix(q, l);
         memcpy(stage.data() + h.off_mem, q->mem, sizeof(int32_t) * (size_t)h.L * h.S);
         d.zcols = nullptr;
         if (h.has_zero) {
@@ -1191,7 +1227,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 GdpDevLayer &y = lay[(size_t)k * g.max_L + l];
                 y.hi = -1;
                 if (l >= h.L) continue;
-                const int mat = q->inter_index ? q->inter_index[l] : l;
+                const int mat = h.matrix(q, l);
                 y.src = d.H + (int64_t)(l % h.nbuf) * d.hstride;
                 y.dst = d.H + (int64_t)((l + 1) % h.nbuf) * d.hstride + h.P;
                 y.ro = d.roff + (int64_t)l * rows;

@@ -69,6 +69,13 @@ def test_layout_audit_through_the_library():
            [(1, 1, 1), (2, 1, 2), (3, 1024, 64), (9, 257, 333), (40, 3, 100001)]]
     for inst in odd:
         _lib.check_layout([prob(inst)])
+    # a dense [L,S,S] array that repeats matrices (they are kept once): runs of equal ones, one that comes
+    # back later, and more different ones than the library looks back at
+    inst = W.random_instance(rng, 24, 5, 300, mem_hi=40)
+    dense = inst.inter[[0, 0, 1, 1, 0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 11, 3, 10, 0, 12, 12, 12, 1, 13]]
+    keys = sorted(inst.other_mem)
+    _lib.check_layout([_lib.Problem(inst.mem, inst.intra, np.ascontiguousarray(dense), inst.V,
+                                    [inst.other_mem[k] for k in keys], [inst.other_time[k] for k in keys])])
     bad = W.random_instance(rng, 3, 4, 50, mem_hi=9)
     with pytest.raises(ValueError):                       # validation comes first: a start row above the table
         _lib.check_layout([_lib.Problem(bad.mem, bad.intra, bad.inter, bad.V, [-1], [0.0])])
