@@ -49,6 +49,13 @@ void make(Case &c, int L, int S, int V, int mem_hi, bool shared, unsigned flags)
     for (auto &x : c.intra) x = rnd_unit() < 0.05 ? INFINITY : 1.0 + 19.0 * rnd_unit();
     for (auto &x : c.inter) x = 5.0 * rnd_unit();
     for (auto &x : c.index) x = rnd_int(0, T - 1);
+    if (!shared && rnd_int(0, 1))   // a dense array as the reference's callers pass it: mostly copies of a few matrices
+        for (int l = 1; l < L; ++l) {
+            const int r = rnd_int(0, 9);
+            const int from = r < 6 ? l - 1 : r < 8 ? rnd_int(0, l - 1) : l;
+            if (from != l)
+                memcpy(c.inter.data() + (size_t)l * S * S, c.inter.data() + (size_t)from * S * S, sizeof(double) * S * S);
+        }
     c.other_mem = {0, V / 64, V / 4, (int64_t)V + 5};
     c.other_time = {0.0, 1.0, 2.0, 3.0};
     c.p = gdp_problem{L, V, S, c.mem.data(), c.intra.data(), c.inter.data(), shared ? c.index.data() : nullptr,
