@@ -18,6 +18,7 @@
 #include <mutex>
 #include <new>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 // ---- shared with gdp_static.hip (declared in gdp_host.h) ---------------------------------------------
@@ -366,6 +367,12 @@ struct HostInst {
     std::vector<int32_t> mat_of;   // layer -> kept matrix
     std::vector<int32_t> mat_src;  // kept matrix -> the layer whose copy is taken
     int matrix(const gdp_problem *q, int l) const { return q->inter_index ? q->inter_index[l] : mat_of[(size_t)l]; }
+    // where the caller keeps kept matrix t
+    const double *matrix_at(const gdp_problem *q, int t) const
+    {
+        return q->inter + (size_t)(q->inter_index ? t : mat_src[(size_t)t]) * (size_t)S * (size_t)S;
+    }
+    int tables_of = -1;   // an earlier instance of the plan (sorted order) whose device copy of the matrices this one reads
 };
 
 // The reference's callers pass one transition matrix per layer, and almost all of them are copies of a
@@ -1053,8 +1060,32 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             }
         g.off_rows = take(sizeof(int32_t) * std::max<size_t>(g.rows.size(), 1));
     }
-    for (auto &h : inst) {
-        h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_PAD) * h.SP);
+    // Instances that were handed the very same transition matrices (same addresses: the instances of a sweep
+    // that differ in their memory and intra costs only, the stages of one pipeline degree) read ONE device
+    // copy: workgroups of different instances that run side by side on a CU then find each other's
+    // transition costs in the scalar cache instead of evicting them.
+    std::unordered_map<const double *, std::vector<int>> owners;   // first kept matrix -> instances with a copy of their own
+    for (size_t i = 0; i < inst.size(); ++i) {
+        HostInst &h = inst[i];
+        const gdp_problem *q = p[h.orig];
+        std::vector<int> &cands = owners[h.matrix_at(q, 0)];
+        h.tables_of = -1;
+        for (int j : cands) {
+            const HostInst &o = inst[(size_t)j];
+            if (o.S != h.S || o.n_inter != h.n_inter || o.SU != h.SU || o.SP != h.SP) continue;
+            bool same = true;
+            for (int t = 1; same && t < h.n_inter; ++t) same = o.matrix_at(p[o.orig], t) == h.matrix_at(q, t);
+            if (same) {
+                h.tables_of = j;
+                break;
+            }
+        }
+        if (h.tables_of >= 0) {
+            h.off_inter = inst[(size_t)h.tables_of].off_inter;
+        } else {
+            h.off_inter = take(sizeof(double) * (size_t)h.n_inter * (h.SU + GDP_SRC_PAD) * h.SP);
+            cands.push_back((int)i);
+        }
         h.off_intra = take(sizeof(double) * (size_t)h.L * h.SP);
         h.off_index = take(sizeof(int32_t) * (size_t)h.L);
         h.off_roff = take(sizeof(int64_t) * (size_t)(h.L + 1) * (h.SU + GDP_SRC_PAD));
@@ -1159,8 +1190,8 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
         // inter: [T][rows][SP], zero padded
         double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
-        for (int t = 0; t < h.n_inter; ++t) {
-            const double *from = q->inter + (size_t)(q->inter_index ? t : h.mat_src[(size_t)t]) * h.S * h.S;
+        for (int t = 0; t < (h.tables_of >= 0 ? 0 : h.n_inter); ++t) {
+            const double *from = h.matrix_at(q, t);
             for (int a = 0; a < h.S; ++a)
                 memcpy(it + ((size_t)t * rows + a) * h.SP, from + (size_t)a * h.S, sizeof(double) * (size_t)h.S);
         }
@@ -1447,7 +1478,15 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
     }
     for (const HostInst &h : pl->inst) {
         const size_t rows = (size_t)h.SU + GDP_SRC_PAD;
-        span(h.off_inter, sizeof(double) * (size_t)h.n_inter * rows * h.SP);
+        if (h.tables_of < 0) {
+            span(h.off_inter, sizeof(double) * (size_t)h.n_inter * rows * h.SP);
+        } else {
+            const int j = h.tables_of;
+            if (j < 0 || j >= pl->n) return bad("owner of shared transition matrices", j, pl->n, 0);
+            const HostInst &o = pl->inst[(size_t)j];
+            if (o.tables_of >= 0 || o.off_inter != h.off_inter || o.n_inter != h.n_inter || o.S != h.S || o.SU != h.SU || o.SP != h.SP)
+                return bad("shared transition matrices", j, (long long)o.off_inter, (long long)h.off_inter);
+        }
         span(h.off_intra, sizeof(double) * (size_t)h.L * h.SP);
         span(h.off_index, sizeof(int32_t) * (size_t)h.L);
         span(h.off_roff, sizeof(int64_t) * (size_t)(h.L + 1) * rows);

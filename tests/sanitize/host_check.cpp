@@ -129,6 +129,21 @@ int main()
             make(c, 5, 44, 3000, 300, false, flags);
             check({&c}, "flags");
         }
+        // instances that point at the same transition matrices (they read one device copy), among others that do not
+        for (int shared = 0; shared < 2; ++shared) {
+            std::vector<Case> cs(7);
+            std::vector<Case *> ptrs;
+            for (size_t k = 0; k < cs.size(); ++k) {
+                make(cs[k], 6, k == 5 ? 22 : 44, 2500, 300, shared != 0, 0);
+                if (k >= 1 && k <= 4 && k != 3) {
+                    cs[k].p.inter = cs[0].p.inter;
+                    cs[k].p.inter_index = cs[0].p.inter_index;
+                    cs[k].p.n_inter = cs[0].p.n_inter;
+                }
+                ptrs.push_back(&cs[k]);
+            }
+            check(ptrs, "batch with shared matrices");
+        }
         if (preset[0]) unsetenv(preset[0]);
         if (lat) unsetenv("GALVATRON_DP_FUSED");
     }

@@ -70,3 +70,43 @@ def test_dense_array_through_the_plugin_signature(golden):
     inst = H.build_case(rec)
     assert inst.inter.shape == (inst.L, inst.S, inst.S)
     H.assert_same_results(H.hip_solve(inst), H.golden_results(rec), "cfg1 dense")
+
+
+def test_instances_of_a_batch_that_were_handed_the_same_matrices(monkeypatch):
+    """Instances that point at the same transition matrices read one device copy: a batch that mixes
+    instances sharing a table (with an index), instances sharing a dense array (one of them a shorter
+    prefix of it), and instances with matrices of their own, under every launch scheme, against the
+    oracle instance by instance."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    rng = np.random.Generator(np.random.PCG64(31))
+    S, V = 12, 900
+    tables = np.ascontiguousarray(rng.uniform(0.0, 6.0, size=(3, S, S)))
+    dense = np.ascontiguousarray(tables[[0, 0, 1, 1, 1, 2]])
+    other = np.ascontiguousarray(rng.uniform(0.0, 6.0, size=(2, S, S)))
+    specs = [("index", tables, [0, 1, 1, 2, 2]), ("index", tables, [2, 2, 0]), ("index", tables, [1, 0, 0, 0, 2, 2, 1]),
+             ("dense", dense, None), ("dense", dense[:4], None), ("dense", dense[:6], None),
+             ("index", other, [0, 1, 0, 1]), ("dense", np.ascontiguousarray(tables[[1, 1, 1]]), None)]
+    probs, wants = [], []
+    for kind, arr, index in specs:
+        L = len(index) if index is not None else arr.shape[0]
+        inst = W.random_instance(rng, L, S, V, mem_hi=V // 6, inf_frac=0.05, n_keys=2)
+        full = arr[index] if index is not None else arr
+        wants.append(O.solve(inst.mem, inst.intra, full, inst.V, inst.other_mem, inst.other_time))
+        keys = sorted(inst.other_mem)
+        om, ot = [inst.other_mem[k] for k in keys], [inst.other_time[k] for k in keys]
+        probs.append((keys, lambda kind=kind, arr=arr, index=index, inst=inst, om=om, ot=ot: _lib.Problem(
+            inst.mem, inst.intra, arr, inst.V, om, ot,
+            inter_index=None if index is None else np.asarray(index, dtype=np.int32))))
+    for env in ({}, {"GALVATRON_DP_FUSED": "1"}, {"GALVATRON_DP_FUSED": "0", "GALVATRON_DP_FLOW": "0"},
+                {"GALVATRON_DP_KEEP_MARKS": "1"}):
+        for k in _PRESETS:
+            monkeypatch.delenv(k, raising=False)
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        built = [make() for _, make in probs]
+        _lib.check_layout(built)
+        _lib.solve_batch(built)
+        for n, ((keys, _), prob, want) in enumerate(zip(probs, built, wants)):
+            H.assert_same_results(_results(prob, keys), want, f"instance {n} {env}")
