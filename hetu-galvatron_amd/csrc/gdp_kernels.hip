@@ -1163,6 +1163,38 @@ __device__ __forceinline__ void wave_argmin(double &val, int &idx)
                            __builtin_amdgcn_readlane(__double2loint(val), 63));
 }
 
+// The wavefront's lowest value, in every lane; same folding as wave_argmin.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void min_step(double &val)
+{
+    const int lo = __double2loint(val), hi = __double2hiint(val);
+    const int olo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+    const int ohi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+    val = min_f64(val, __hiloint2double(ohi, olo));
+}
+
+__device__ __forceinline__ double wave_min(double val)
+{
+    min_step<0x111, 0xf>(val);
+    min_step<0x112, 0xf>(val);
+    min_step<0x114, 0xf>(val);
+    min_step<0x118, 0xf>(val);
+    min_step<0x142, 0xa>(val);
+    min_step<0x143, 0xc>(val);
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(val), 63),
+                            __builtin_amdgcn_readlane(__double2loint(val), 63));
+}
+
+// Lane s holds candidate s (+inf in lanes that hold none): the lowest index among the lowest candidates
+// -- the lowest lane whose value equals the wavefront's minimum; lane 0 when all are +inf.  A third of
+// the instructions of the reduction over (value, index) pairs.
+__device__ __forceinline__ int wave_argmin_by_lane(double val)
+{
+    const double lowest = wave_min(val);
+    const unsigned long long eq = __builtin_amdgcn_ballot_w64(val == lowest);
+    return eq ? (int)__builtin_ctzll(eq) : 64;   // (no lane equals the minimum only if the values are NaN)
+}
+
 // Epilogue of csrc/dp_core.cpp:78-117 for one key per wavefront: first argmin of the start row,
 // then the dependent walk back through the layers.  MARKS: the walk reads the stored argmin table.
 // Otherwise every cost buffer of the run is still there, and the wavefront recomputes the argmin of
@@ -1234,43 +1266,56 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
             // offset, intra cost -- fetched one layer ahead, so that the step from a cell to its
             // predecessor is a lane read, one round of gathered loads (cost row and transition column
             // together) and the reduction, instead of a dependent scalar load before the gather.
+            // The one wavefront is bound by its own chain of instructions as much as by the round trip, so the
+            // step is kept short: the addresses move by a stride per layer instead of being multiplied out, and
+            // the reduction is over values only (wave_argmin_by_lane).
             const int sl = lane < S ? lane : S - 1;
-            int m_next = mem[(int64_t)i * S + sl];
-            int64_t r_next = roff[(int64_t)i * rows + sl];
-            double a_next = intra[(int64_t)i * SP + sl];
-            int t_next = uload(inter_index + i);
+            const int32_t *mem_p = mem + (int64_t)i * S + sl;          // layer i, this lane's strategy
+            const int64_t *roff_p = roff + (int64_t)i * rows + sl;
+            const double *intra_p = intra + (int64_t)i * SP + sl;
+            const int32_t *index_p = inter_index + i;
+            const double *inter_lane = inter + (int64_t)sl * SP;      // row `lane` of matrix 0
+            const int64_t mat_stride = (int64_t)rows * SP;
+            int b = i % nbuf;                                         // the cost buffer that holds the costs before layer i
+            const double *src = H + (int64_t)b * hstride;
+            int m_next = *mem_p;
+            int64_t r_next = *roff_p;
+            double a_next = *intra_p;
+            int64_t t_next = uload(index_p) * mat_stride;
             for (; i > 0; --i) {
                 const int cur = idx;
                 const int m_cur = m_next;
                 const int64_t r_cur = r_next;
                 const double a_cur = a_next;
-                const int t_cur = t_next;
+                const int64_t t_cur = t_next;
                 if (i > 1) {
-                    m_next = mem[(int64_t)(i - 1) * S + sl];
-                    r_next = roff[(int64_t)(i - 1) * rows + sl];
-                    a_next = intra[(int64_t)(i - 1) * SP + sl];
-                    t_next = uload(inter_index + (i - 1));
+                    mem_p -= S;
+                    roff_p -= rows;
+                    intra_p -= SP;
+                    index_p -= 1;
+                    m_next = *mem_p;
+                    r_next = *roff_p;
+                    a_next = *intra_p;
+                    t_next = uload(index_p) * mat_stride;
                 }
                 const int m_here = __builtin_amdgcn_readlane(m_cur, cur);
                 v -= m_here;  // the source row of cell (i, v, cur)
                 if (v < 0) break;
-                const double *src = H + (int64_t)(i % nbuf) * hstride;  // costs before layer i
                 const double a = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(a_cur), cur),
                                                   __builtin_amdgcn_readlane(__double2loint(a_cur), cur));
                 double bv = INFINITY;
-                int bi = 0x7fffffff;
                 if (lane < S) {
                     // a cell with mem == 0 took its lower strategies from its own layer (gdp_launch_zero_pass)
                     const double x = (m_here == 0 && lane < cur)
                                          ? H[(int64_t)((i + 1) % nbuf) * hstride + roff[(int64_t)(i + 1) * rows + lane] + v]
                                          : src[r_cur + v];
-                    bv = (x + inter[((int64_t)t_cur * rows + lane) * SP + cur]) + a;
-                    bi = lane;
+                    bv = (x + inter_lane[t_cur + cur]) + a;
                 }
-                wave_argmin(bv, bi);
-                idx = __builtin_amdgcn_readfirstlane(bi);
+                idx = wave_argmin_by_lane(bv);
                 if (idx >= S) { v = -1; break; }
                 if (lane == 0) path[i - 1] = idx;
+                if (--b < 0) b = nbuf - 1;
+                src = H + (int64_t)b * hstride;
             }
             i = 0;
         }
