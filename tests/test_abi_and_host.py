@@ -103,3 +103,25 @@ def test_problem_shape_checks():
     p = _lib.Problem(np.ones((2, 3), np.int32), np.ones((2, 3)), np.zeros((1, 3, 3)), 10, [0], [0.0],
                      inter_index=[0, 0])
     assert p.relaxations == 2 * 10 * 9
+
+
+def test_problem_points_at_the_arrays_it_keeps():
+    """The C structure of a problem holds the addresses of the arrays the Python object keeps alive --
+    also for arrays that do not allow a writable view (read-only inputs) and for key lists of length
+    zero, where the address comes from another route."""
+    mem = np.arange(6, dtype=np.int32).reshape(2, 3) + 1
+    intra = np.ones((2, 3))
+    inter = np.zeros((2, 3, 3))
+    for a in (mem, intra, inter):
+        a.setflags(write=False)
+    p = _lib.Problem(mem, intra, inter, 10, [0, 3], [0.0, 1.0])
+    c = p._c_problem
+    addr = lambda a: a.__array_interface__["data"][0]      # noqa: E731
+    assert (c.mem, c.intra, c.inter) == (addr(p.mem), addr(p.intra), addr(p.inter))
+    assert p.mem is mem and p.intra is intra and p.inter is inter      # no copies of arrays that already fit
+    assert (c.other_mem, c.other_time) == (addr(p.other_mem), addr(p.other_time))
+    r = p._c_result
+    assert (r.total, r.remaining, r.res) == (addr(p.total), addr(p.remaining), addr(p.res))
+    assert list(p.total) == [np.inf, np.inf] and list(p.remaining) == [-1, -1] and (p.res == -1).all()
+    q = _lib.Problem(mem.copy(), intra.copy(), inter.copy(), 10, [], [])
+    assert q.n_key == 0 and q.total.shape == (0,)
