@@ -1168,7 +1168,67 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // the buffer any more
         memset(stage.p, 0, small_bytes);
     }
+    // {tiles a reader reaches down, first tile to compute, last tile to compute} per layer
     std::vector<std::vector<int32_t>> h_band((size_t)n);
+    for (int i = 0; i < n; ++i) {
+        const HostInst &h = inst[(size_t)i];
+        h_band[(size_t)i].assign((size_t)h.L * 3, 0);
+        fill_bands(p[h.orig], h, 64 * GDP_VARIANTS[h.variant].r, pl->skip, h_band[(size_t)i].data(), &pl->executed,
+                   pl->flow_ready);
+    }
+    // Rows of a layer's output below its band are +inf and are filled once per plan -- those that something
+    // reads: the band of the next layer reaches down by at most this layer's largest memory cost (the
+    // backtrack reads what the relaxation read), the epilogue and the pass for memory costs of 0 read anywhere.
+    auto fill_from_of = [&](int i, int l) -> int32_t {
+        const HostInst &h = inst[(size_t)i];
+        if (l + 1 >= h.L || h.has_zero) return 0;
+        const int64_t lo_next = h_band[(size_t)i][3 * (size_t)(l + 1) + 1];
+        const int64_t reach = (int64_t)h_band[(size_t)i][3 * (size_t)l];   // tiles
+        return (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
+    };
+    // A small plan laid out for the flow launch, the turn free right now (its first run will most likely
+    // flow): the kernel that prepares its cost buffers -- pads, zeros, the filled rows, NaN into the bands --
+    // gets what it needs with its arguments and starts here, before the tables below have even been built;
+    // it runs beside the host's work on them and beside their upload (which then goes over the second stream
+    // in one piece).  (A Galvatron-like call: upload 15 us, then this kernel 42 us, then the first launch;
+    // now the kernel is under way 30 us earlier.)
+    bool turn_free = false;
+    if (!pl->dry && pl->flow_ready) {
+        std::lock_guard<std::mutex> lk(g_fused_mu);
+        turn_free = !g_fused_busy;
+    }
+    bool prepared_early = false;
+    if (turn_free && n <= GDP_PREP_MAX_INST) {
+        int layers = 0;
+        for (const auto &h : inst) layers += h.L;
+        if (layers <= GDP_PREP_MAX_LAYERS) {
+            GdpPrepArgs A;
+            memset(&A, 0, sizeof A);
+            int e = 0;
+            for (int i = 0; i < n; ++i) {
+                const HostInst &h = inst[(size_t)i];
+                GdpPrepArgs::Inst &a = A.inst[i];
+                a.H = reinterpret_cast<double *>(pl->dbase + h.off_H);
+                a.hstride = (int64_t)(h.S + 1) * h.ld;
+                a.ld = h.ld;
+                a.P = h.P;
+                a.S = h.S;
+                a.L = h.L;
+                a.tile_rows = 64 * GDP_VARIANTS[h.variant].r;
+                a.first_layer = e;
+                for (int l = 0; l < h.L; ++l, ++e) {
+                    A.lo[e] = h_band[(size_t)i][3 * (size_t)l + 1];
+                    A.hi[e] = h_band[(size_t)i][3 * (size_t)l + 2];
+                    A.fill_from[e] = fill_from_of(i, l);
+                }
+            }
+            A.abort_flag = reinterpret_cast<int32_t *>(pl->dbase + pl->off_abort);
+            A.n_inst = n;
+            A.nan_bands = 1;
+            GDP_HIP(gdp_launch_prepare_args(A, pl->stream));
+            prepared_early = true;
+        }
+    }
     GdpDevInst *di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
     GdpDevKey *dk = reinterpret_cast<GdpDevKey *>(stage.data() + pl->off_keys);
     for (int i = 0; i < n; ++i) {
@@ -1187,7 +1247,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         d.ld = h.ld; d.ldm = h.ldm;
         d.L = h.L; d.V = h.V; d.S = h.S; d.SP = h.SP; d.SU = h.SU; d.P = h.P; d.ntile = h.ntile;
         const int rows = h.SU + GDP_SRC_PAD;  // source rows per matrix / offsets per layer
-        const int tile_rows = 64 * GDP_VARIANTS[h.variant].r;
         // inter: [T][rows][SP], zero padded
         double *it = reinterpret_cast<double *>(stage.data() + h.off_inter);
         for (int t = 0; t < (h.tables_of >= 0 ? 0 : h.n_inter); ++t) {
@@ -1227,9 +1286,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             }
             for (int s = h.S; s < rows; ++s) row[s] = inf_row;  // padding sources and prefetch targets
         }
-        // {tiles a reader reaches down, first tile to compute, last tile to compute} per layer
-        h_band[(size_t)i].assign((size_t)h.L * 3, 0);
-        fill_bands(q, h, tile_rows, pl->skip, h_band[(size_t)i].data(), &pl->executed, pl->flow_ready);
         for (int k = 0; k < h.n_key; ++k) {
             GdpDevKey &key = dk[h.key_begin + k];
             key.other_mem = q->other_mem[k];
@@ -1281,16 +1337,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                         }
                         y.gate |= (uint32_t)best_s << (8 * part);
                     }
-                // Rows of this layer's output below its band are +inf and are filled once per plan -- those that
-                // something reads: the band of the next layer reaches down by at most this layer's largest
-                // memory cost (the backtrack reads what the relaxation read), the epilogue and the pass for
-                // memory costs of 0 read anywhere.
-                y.fill_from = 0;
-                if (l + 1 < h.L && !h.has_zero) {
-                    const int64_t lo_next = h_band[(size_t)(g.first + k)][3 * (size_t)(l + 1) + 1];
-                    const int64_t reach = (int64_t)h_band[(size_t)(g.first + k)][3 * (size_t)l];   // tiles
-                    y.fill_from = (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
-                }
+                y.fill_from = fill_from_of(g.first + k, l);
                 y.dep = h_band[(size_t)(g.first + k)][3 * (size_t)l];
                 if ((int64_t)h_band[(size_t)(g.first + k)][3 * (size_t)l + 1] * (64 * GDP_VARIANTS[h.variant].r) > y.fill_from)
                     g.any_fill = true;
@@ -1397,16 +1444,16 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // the per-instance inputs follow on a second stream, beside that kernel.
     size_t tables_bytes = small_bytes;
     bool &split_upload = pl->split_upload;
-    {
-        std::lock_guard<std::mutex> lk(g_fused_mu);
-        split_upload = pl->flow_ready && !g_fused_busy;
-    }
-    if (split_upload) {
+    split_upload = turn_free;
+    if (prepared_early) {
+        tables_bytes = 0;      // everything over the second stream, beside the kernel that is already running
+    } else if (split_upload) {
         for (const auto &h : inst) tables_bytes = std::min(tables_bytes, h.off_inter);
         split_upload = tables_bytes > 0 && tables_bytes < small_bytes;
     }
-    GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), split_upload ? tables_bytes : small_bytes, hipMemcpyHostToDevice,
-                           pl->stream));
+    if (!prepared_early)
+        GDP_HIP(hipMemcpyAsync(pl->dbase, stage.data(), split_upload ? tables_bytes : small_bytes, hipMemcpyHostToDevice,
+                               pl->stream));
     if (split_upload) {
         // (the side stream is idle: whatever it last carried was joined to a main stream that has been waited for)
         GDP_HIP(hipMemcpyAsync(pl->dbase + tables_bytes, stage.data() + tables_bytes, small_bytes - tables_bytes,
@@ -1420,6 +1467,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // taken every time never pays for it.
         const bool nan_bands = split_upload;
         for (const Group &g : pl->groups) {
+            if (prepared_early) continue;
             if (!nan_bands)   // (one launch instead of three pays only where the three are short)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                         64 * GDP_VARIANTS[g.variant].r,

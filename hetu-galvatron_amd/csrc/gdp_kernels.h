@@ -177,6 +177,23 @@ hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t ma
 // launch, and, with nan_bands, what gdp_launch_flow_reset does as well.
 hipError_t gdp_launch_prepare(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
                               int max_L, int tile_rows, bool nan_bands, int32_t *abort_flag, hipStream_t stream);
+// The same from the kernel's own arguments, for a few small instances (no table of the plan has to be on
+// the device yet): per instance where its cost buffers lie, per layer -- `first_layer` of an instance on --
+// the band and the first filled row of its output.
+#define GDP_PREP_MAX_INST 16
+#define GDP_PREP_MAX_LAYERS 224
+struct GdpPrepArgs {
+    struct Inst {
+        double *H;
+        int64_t hstride, ld, P;
+        int32_t S, L, tile_rows, first_layer;
+    } inst[GDP_PREP_MAX_INST];
+    int32_t lo[GDP_PREP_MAX_LAYERS], hi[GDP_PREP_MAX_LAYERS], fill_from[GDP_PREP_MAX_LAYERS];
+    int32_t *abort_flag;
+    int32_t n_inst, nan_bands;
+};
+static_assert(sizeof(GdpPrepArgs) <= 3584, "passed by value with the kernel arguments");
+hipError_t gdp_launch_prepare_args(const GdpPrepArgs &A, hipStream_t stream);
 #define GDP_INIT_PADS 1
 #define GDP_INIT_ZERO 2
 #define GDP_INIT_POISON 4

@@ -1017,6 +1017,32 @@ __global__ __launch_bounds__(256) void gdp_fill_kernel(const GdpDevInst *__restr
 // initial f), +inf in the rows below the band of every layer's output that something reads, and -- with
 // `nan_bands`, for a plan that will run as a flow launch -- NaN in the bands.
 // grid = (x chunks, rows 0..S, instances x (max_L + 1) buffers).
+// Row `row` of one cost buffer (h: its first element, pad included): the output of a layer whose band is
+// [lo, hi] tiles and whose rows from fill_from up to the band are read by something -- or, `whole`, buffer 0
+// (zeros behind the pad) or the +inf row of any buffer.
+__device__ __forceinline__ void prepare_row(double *h, bool whole, bool inf_row, int64_t ld, int64_t P, int lo, int hi,
+                                            int64_t fill_from, int tile_rows, int nan_bands)
+{
+    const double inf = INFINITY;
+    const double nan = __builtin_nan("");
+    if (whole) {
+        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ld; i += (int64_t)gridDim.x * blockDim.x)
+            h[i] = (inf_row || i < P) ? inf : 0.0;
+        return;
+    }
+    int64_t band_from = (int64_t)lo * tile_rows;
+    int64_t band_to = hi >= lo ? (int64_t)(hi + 1) * tile_rows : band_from;
+    if (band_from > ld - P) band_from = ld - P;
+    if (band_to > ld - P) band_to = ld - P;
+    // the pad, then rows fill_from .. end of what is written (nothing in between is touched)
+    const int64_t end = nan_bands ? band_to : band_from;
+    const int64_t n = P + (end > fill_from ? end - fill_from : 0);
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t u = j < P ? j - P : j - P + fill_from;
+        h[P + u] = (u < band_from) ? inf : nan;
+    }
+}
+
 __global__ __launch_bounds__(256) void gdp_prepare_kernel(const GdpDevInst *__restrict__ insts,
                                                           const GdpDevLayer *__restrict__ lay, int max_L, int tile_rows,
                                                           int nan_bands, int32_t *abort_flag)
@@ -1030,30 +1056,43 @@ __global__ __launch_bounds__(256) void gdp_prepare_kernel(const GdpDevInst *__re
     const int64_t ld = uload(&I->ld);
     const int64_t P = uload(&I->P);
     double *h = uload(&I->H) + (int64_t)b * uload(&I->hstride) + (int64_t)row * ld;
-    int64_t fill_from = 0, band_from = 0, band_to = 0;   // rows of this buffer (layer b - 1's output)
+    int lo = 0, hi = -1;
+    int64_t fill_from = 0;   // rows of this buffer (layer b - 1's output)
     if (b >= 1) {
         const GdpDevLayer *Y = lay + ((int64_t)inst * max_L + (b - 1));
-        const int lo = uload(&Y->lo), hi = uload(&Y->hi);
+        lo = uload(&Y->lo);
+        hi = uload(&Y->hi);
         fill_from = uload(&Y->fill_from);
-        band_from = (int64_t)lo * tile_rows;
-        band_to = hi >= lo ? (int64_t)(hi + 1) * tile_rows : band_from;
-        if (band_from > ld - P) band_from = ld - P;
-        if (band_to > ld - P) band_to = ld - P;
     }
-    const double inf = INFINITY;
-    const double nan = __builtin_nan("");
-    if (row == S || b == 0) {   // the whole row
-        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ld; i += (int64_t)gridDim.x * blockDim.x)
-            h[i] = (row == S || i < P) ? inf : 0.0;
-        return;
+    prepare_row(h, row == S || b == 0, row == S, ld, P, lo, hi, fill_from, tile_rows, nan_bands);
+}
+
+// The same for a few small instances, everything it needs in its arguments: it can then run before the
+// plan's tables have been uploaded, beside their upload (and beside the host's work on them).
+// grid = (x chunks, rows 0..max S, buffers of all instances).
+__global__ __launch_bounds__(256) void gdp_prepare_args_kernel(const GdpPrepArgs A)
+{
+    if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) *A.abort_flag = 0;
+    int inst = 0, b = (int)blockIdx.z;     // buffer b of instance inst
+    while (inst + 1 < A.n_inst && b > A.inst[inst].L) {
+        b -= A.inst[inst].L + 1;
+        ++inst;
     }
-    // the pad, then rows fill_from .. end of what is written (nothing in between is touched)
-    const int64_t end = nan_bands ? band_to : band_from;
-    const int64_t n = P + (end > fill_from ? end - fill_from : 0);
-    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t u = j < P ? j - P : j - P + fill_from;
-        h[P + u] = (u < band_from) ? inf : nan;
+    const int S = A.inst[inst].S, L = A.inst[inst].L;
+    const int row = blockIdx.y;
+    if (b > L || row > S) return;
+    const int64_t ld = A.inst[inst].ld;
+    const int64_t P = A.inst[inst].P;
+    double *h = A.inst[inst].H + (int64_t)b * A.inst[inst].hstride + (int64_t)row * ld;
+    int lo = 0, hi = -1;
+    int64_t fill_from = 0;
+    if (b >= 1) {
+        const int e = A.inst[inst].first_layer + (b - 1);
+        lo = A.lo[e];
+        hi = A.hi[e];
+        fill_from = A.fill_from[e];
     }
+    prepare_row(h, row == S || b == 0, row == S, ld, P, lo, hi, fill_from, A.inst[inst].tile_rows, A.nan_bands);
 }
 
 __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restrict__ insts, int what)
@@ -1525,6 +1564,26 @@ hipError_t gdp_launch_prepare(const GdpDevInst *insts, int n_inst, int64_t max_l
         hipLaunchKernelGGL(gdp_prepare_kernel, dim3(bx, (unsigned)(max_S + 1), (unsigned)(n * (max_L + 1))), dim3(256), 0,
                            stream, insts + i0, lay + (int64_t)i0 * max_L, max_L, tile_rows, nan_bands ? 1 : 0, abort_flag);
     }
+    return hipGetLastError();
+}
+
+hipError_t gdp_launch_prepare_args(const GdpPrepArgs &A, hipStream_t stream)
+{
+    if (A.n_inst < 1 || A.n_inst > GDP_PREP_MAX_INST) return hipErrorInvalidValue;
+    int64_t max_ld = 0;
+    int max_S = 0, buffers = 0, layers = 0;
+    for (int i = 0; i < A.n_inst; ++i) {
+        if (A.inst[i].L < 1 || A.inst[i].first_layer != layers) return hipErrorInvalidValue;
+        max_ld = A.inst[i].ld > max_ld ? A.inst[i].ld : max_ld;
+        max_S = A.inst[i].S > max_S ? A.inst[i].S : max_S;
+        buffers += A.inst[i].L + 1;
+        layers += A.inst[i].L;
+    }
+    if (layers > GDP_PREP_MAX_LAYERS) return hipErrorInvalidValue;
+    unsigned bx = (unsigned)((max_ld + 256 * 4 - 1) / (256 * 4));
+    if (bx == 0) bx = 1;
+    if (bx > 64u) bx = 64u;
+    hipLaunchKernelGGL(gdp_prepare_args_kernel, dim3(bx, (unsigned)(max_S + 1), (unsigned)buffers), dim3(256), 0, stream, A);
     return hipGetLastError();
 }
 

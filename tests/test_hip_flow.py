@@ -289,3 +289,30 @@ def test_flow_launch_on_the_fuzz_shapes_without_exports():
                     flowed += t.flow
                     H.assert_same_results(_results(prob, keys), (wt, wr, wm), f"shape {(L, S, V)} variant {variant} run {rep}")
     assert flowed > len(SHAPES)
+
+
+def test_small_plans_on_both_sides_of_the_early_preparation():
+    """Up to 16 instances with up to 224 layers in all get their cost buffers prepared by a kernel that is
+    fed with its arguments and starts before the plan's tables are uploaded; one more instance or layer
+    takes the ordinary way.  One-shot solves (gdp_solve_batch) on both sides of both limits, twice each
+    (the second lands in the memory the first left behind), against the oracle."""
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    from oracle import dp_oracle as O
+    rng = np.random.Generator(np.random.PCG64(5))
+
+    def batch(shapes):
+        insts = [W.random_instance(rng, L, S, V, mem_hi=max(2, V // (L + 2)), inf_frac=0.05, n_keys=2) for (L, S, V) in shapes]
+        wants = [O.solve(i.mem, i.intra, i.inter, i.V, i.other_mem, i.other_time) for i in insts]
+        for rep in range(2):
+            probs = [_problem(i) for i in insts]
+            _lib.solve_batch(probs)
+            for n, (i, prob, want) in enumerate(zip(insts, probs, wants)):
+                H.assert_same_results(_results(prob, sorted(i.other_mem)), want, f"{len(shapes)} instances, #{n}, run {rep}")
+
+    batch([(224, 5, 700)])
+    batch([(225, 5, 700)])
+    batch([(14, 9, 400)] * 16)                      # 16 instances, 224 layers
+    batch([(14, 9, 400)] * 15 + [(15, 9, 400)])     # 225 layers
+    batch([(6, 12, 300)] * 17)
+    batch([(3, 22, 900), (40, 8, 500), (1, 13, 200), (28, 40, 2000)])
