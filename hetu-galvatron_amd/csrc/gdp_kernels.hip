@@ -1344,17 +1344,21 @@ __global__ __launch_bounds__(64) void gdp_epilogue_kernel(const GdpDevInst *__re
                                                   __builtin_amdgcn_readlane(__double2loint(a_cur), cur));
                 double bv = INFINITY;
                 if (lane < S) {
+                    double x = src[r_cur + v];
                     // a cell with mem == 0 took its lower strategies from its own layer (gdp_launch_zero_pass)
-                    const double x = (m_here == 0 && lane < cur)
-                                         ? H[(int64_t)((i + 1) % nbuf) * hstride + roff[(int64_t)(i + 1) * rows + lane] + v]
-                                         : src[r_cur + v];
+                    if (m_here == 0 && lane < cur)
+                        x = H[(int64_t)((i + 1) % nbuf) * hstride + roff[(int64_t)(i + 1) * rows + lane] + v];
                     bv = (x + inter_lane[t_cur + cur]) + a;
                 }
                 idx = wave_argmin_by_lane(bv);
                 if (idx >= S) { v = -1; break; }
                 if (lane == 0) path[i - 1] = idx;
-                if (--b < 0) b = nbuf - 1;
-                src = H + (int64_t)b * hstride;
+                if (--b < 0) {
+                    b = nbuf - 1;
+                    src = H + (int64_t)b * hstride;
+                } else {
+                    src -= hstride;
+                }
             }
             i = 0;
         }
