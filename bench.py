@@ -293,7 +293,8 @@ def main() -> int:
             i0 = insts[0]
             res = {k: np.full(i0.L, -1, dtype=np.int32) for k in i0.other_mem}
             inter = np.ascontiguousarray(i0.inter)
-            args = (i0.L, i0.V, i0.S, i0.mem, None, None, inter, i0.intra, i0.other_mem, i0.other_time, res)
+            f = np.zeros((i0.V, i0.S))              # DPAlg's ``_f`` (dynamic_programming.py:16); ``_mark`` is never read
+            args = (i0.L, i0.V, i0.S, i0.mem, None, f, inter, i0.intra, i0.other_mem, i0.other_time, res)
             times = []
             for _ in range(1 + max(5, min(steps, 30))):
                 h0 = time.perf_counter()

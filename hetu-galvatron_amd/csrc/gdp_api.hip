@@ -373,6 +373,10 @@ struct HostInst {
         return q->inter + (size_t)(q->inter_index ? t : mat_src[(size_t)t]) * (size_t)S * (size_t)S;
     }
     int tables_of = -1;   // an earlier instance of the plan (sorted order) whose device copy of the matrices this one reads
+    // The caller's initial costs where they are not all zero (gdp_problem.f0), one row per strategy -- the
+    // layout of a cost buffer; kept for the life of the plan, because a plan with two cost buffers writes
+    // over buffer 0 in every run and gets them uploaded again before the next.
+    std::vector<double> f0t;
 };
 
 // The reference's callers pass one transition matrix per layer, and almost all of them are copies of a
@@ -558,6 +562,60 @@ struct gdp_plan {
     size_t dry_lds_per_cu = 0;
 };
 
+// The caller's initial costs (gdp_problem.f0): *live says whether anything but +0.0 is in there (an array of
+// zeros is what every caller of the reference passes, and is treated like no array), *maxabs the largest
+// finite magnitude.  The common case is one pass over the array that ORs its words.
+static int scan_f0(const gdp_problem *p, bool *live, double *maxabs)
+{
+    *live = false;
+    *maxabs = 0;
+    if (!p->f0) return 0;
+    const size_t n = (size_t)p->V * (size_t)p->S;
+    uint64_t any = 0;
+    size_t k = 0;
+    for (; k + 64 <= n && !any; k += 64)
+        for (int j = 0; j < 64; ++j) {
+            uint64_t w;
+            memcpy(&w, p->f0 + k + j, sizeof w);
+            any |= w;
+        }
+    for (; k < n && !any; ++k) {
+        uint64_t w;
+        memcpy(&w, p->f0 + k, sizeof w);
+        any |= w;
+    }
+    if (!any) return 0;
+    *live = true;
+    double m = 0;
+    for (k = 0; k < n; ++k) {
+        const double x = p->f0[k];
+        if (x != x || x == -INFINITY) return 1;
+        if (x == 0 && std::signbit(x)) return 2;
+        if (x != INFINITY) m = std::max(m, std::fabs(x));
+    }
+    *maxabs = m;
+    return 0;
+}
+
+// The magnitudes of the cost arrays may add up to COST_BOUND and those of the initial costs reach it, so that
+// no partial sum can overflow.
+static constexpr double COST_BOUND = 5e299;
+
+int gdp_validate_f0(const gdp_problem *p, int i, bool *f0_live)
+{
+    char buf[200];
+    bool live = false;
+    double m = 0;
+    const int what = scan_f0(p, &live, &m);
+    if (f0_live) *f0_live = live;
+    if (what == 0 && m < COST_BOUND) return GDP_OK;
+    snprintf(buf, sizeof buf, "instance %d: %s", i,
+             what == 1 ? "NaN or -inf in f0"
+             : what == 2 ? "-0.0 in f0 (the sign of a zero cost would depend on the order of evaluation)"
+                         : "cost magnitudes could overflow binary64 (f0)");
+    return gdp_fail(what == 2 ? GDP_E_BADARG : GDP_E_NONFINITE, buf);
+}
+
 int gdp_validate(const gdp_problem *p, int i)
 {
     char buf[160];
@@ -633,13 +691,34 @@ int gdp_validate(const gdp_problem *p, int i)
         // reference reads out of bounds; an entry above V-1 is an infeasible key and is answered as such
         if (p->other_mem[k] < 0) return bad(GDP_E_BADARG, "negative other_mem entry (start row above the table)");
     }
-    if (!(bound < 1e300)) return bad(GDP_E_NONFINITE, "cost magnitudes could overflow binary64");
+    if (!(bound < COST_BOUND)) return bad(GDP_E_NONFINITE, "cost magnitudes could overflow binary64");
     return GDP_OK;
 }
 
 namespace {
 
-int validate(const gdp_problem *p, int i) { return gdp_validate(p, i); }
+// Looks through the initial costs of all problems; f0_live[i] != 0 where problem i brings some other than zeros.
+int validate_f0_all(int32_t n, const gdp_problem *const *p, std::vector<char> &f0_live)
+{
+    f0_live.assign((size_t)n, 0);
+    for (int i = 0; i < n; ++i) {
+        bool live = false;
+        const int rc = gdp_validate_f0(p[i], i, &live);
+        if (rc != GDP_OK) return rc;
+        f0_live[(size_t)i] = live ? 1 : 0;
+    }
+    return GDP_OK;
+}
+
+// Validates all problems, initial costs included.
+int validate_all(int32_t n, const gdp_problem *const *p, std::vector<char> &f0_live)
+{
+    for (int i = 0; i < n; ++i) {
+        const int rc = gdp_validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+    }
+    return validate_f0_all(n, p, f0_live);
+}
 
 void destroy(gdp_plan *pl)
 {
@@ -732,7 +811,21 @@ size_t footprint(const gdp_problem *q)
 // the caller starts over with force_marks, i.e. two cost buffers and the argmin table.
 constexpr int GDP_RETRY_WITH_MARKS = 1 << 20;
 
-int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks)
+// The initial costs of the instances that brought some, into the data region of their buffer 0 (behind
+// whatever zeroed it on the plan's stream).
+int upload_f0(gdp_plan *pl)
+{
+    for (const HostInst &h : pl->inst) {
+        if (h.f0t.empty()) continue;
+        double *dst = reinterpret_cast<double *>(pl->dbase + h.off_H) + h.P;
+        GDP_HIP(hipMemcpy2DAsync(dst, sizeof(double) * (size_t)h.ld, h.f0t.data(), sizeof(double) * (size_t)h.V,
+                                 sizeof(double) * (size_t)h.V, (size_t)h.S, hipMemcpyHostToDevice, pl->stream));
+    }
+    return GDP_OK;
+}
+
+// f0_live: null, or per problem whether its f0 holds anything but zeros (validate_all).
+int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks, const char *f0_live)
 {
     pl->n = n;
     if (!pl->dry) GDP_HIP(hipGetDevice(&pl->device));
@@ -816,6 +909,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             if (q->mem[k] == 0) h.has_zero = true;
         }
         h.P = (int)align_up((size_t)std::max(maxm, 1), 64);
+        if (f0_live && f0_live[i] && q->f0 && !pl->dry) {   // [V][S] -> one row per strategy
+            h.f0t.resize((size_t)q->S * (size_t)q->V);
+            for (int v = 0; v < q->V; ++v)
+                for (int s2 = 0; s2 < q->S; ++s2) h.f0t[(size_t)s2 * q->V + v] = q->f0[(size_t)v * q->S + s2];
+        }
     }
     // group by S, then by L descending (stable, so equal shapes keep the caller's order)
     std::stable_sort(inst.begin(), inst.end(), [](const HostInst &a, const HostInst &b) {
@@ -1483,7 +1581,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
     pl->inst.swap(inst);
-    return GDP_OK;
+    return upload_f0(pl);
 }
 
 
@@ -1731,6 +1829,10 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             for (const Group &g : pl->groups)
                 GDP_HIP(gdp_launch_init(d_insts + g.first, g.count, g.max_ld, g.S, g.sched.lay, g.max_L,
                                         64 * GDP_VARIANTS[g.variant].r, g.any_fill ? what : (what & ~GDP_INIT_FILL), pl->stream));
+        if (pl->rezero) {
+            const int rc = upload_f0(pl);
+            if (rc != GDP_OK) return rc;
+        }
     }
     size_t li = 0;
 
@@ -1769,7 +1871,8 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                                          reinterpret_cast<const GdpDevLayer *>(pl->dbase + g.off_lay), g.max_L,
                                          g.active[(size_t)l], g.max_ntile, g.SP, l, pl->stream));
                 if (g.zero_layer[(size_t)l])
-                    GDP_HIP(gdp_launch_zero_pass(pl->keep_marks, d_insts + g.first, g.active[(size_t)l], g.max_V, l, pl->stream));
+                    GDP_HIP(gdp_launch_zero_pass(pl->keep_marks, d_insts + g.first, g.sched.lay, g.max_L,
+                                                 64 * GDP_VARIANTS[g.variant].r, g.active[(size_t)l], g.max_V, l, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
             }
@@ -1912,8 +2015,8 @@ int fetch(gdp_plan *pl, gdp_result *const *r)
     return GDP_OK;
 }
 
-// A plan for problems that validate() has accepted.
-int create_checked(int32_t n, const gdp_problem *const *p, gdp_plan **out)
+// A plan for problems that validate_all() has accepted.
+int create_checked(int32_t n, const gdp_problem *const *p, const char *f0_live, gdp_plan **out)
 {
     *out = nullptr;
     for (int attempt = 0; attempt < 2; ++attempt) {
@@ -1921,7 +2024,7 @@ int create_checked(int32_t n, const gdp_problem *const *p, gdp_plan **out)
         if (!pl) return fail(GDP_E_NOMEM, "plan allocation failed");
         int rc;
         try {
-            rc = create(n, p, pl, attempt == 1);
+            rc = create(n, p, pl, attempt == 1, f0_live);
         } catch (const std::bad_alloc &) {
             rc = fail(GDP_E_NOMEM, "host allocation failed");
         }
@@ -1946,11 +2049,14 @@ int gdp_plan_create(int32_t n, const gdp_problem *const *p, gdp_plan **out)
     *out = nullptr;
     if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
     if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
-    for (int i = 0; i < n; ++i) {
-        int rc = validate(p[i], i);
+    try {
+        std::vector<char> f0_live;
+        const int rc = validate_all(n, p, f0_live);
         if (rc != GDP_OK) return rc;
+        return create_checked(n, p, f0_live.data(), out);
+    } catch (const std::bad_alloc &) {
+        return fail(GDP_E_NOMEM, "host allocation failed");
     }
-    return create_checked(n, p, out);
 }
 
 int gdp_plan_run(gdp_plan *plan, int32_t timing_mode, gdp_timing *timing)
@@ -2011,7 +2117,8 @@ int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_c
     if (n > 65535) return fail(GDP_E_BADARG, "at most 65535 instances per plan");
     if (num_cu < 1 || lds_per_cu < 0) return fail(GDP_E_BADARG, "bad device description");
     for (int i = 0; i < n; ++i) {
-        const int rc = validate(p[i], i);
+        int rc = gdp_validate(p[i], i);
+        if (rc == GDP_OK) rc = gdp_validate_f0(p[i], i, nullptr);
         if (rc != GDP_OK) return rc;
     }
     for (int attempt = 0; attempt < 2; ++attempt) {     // costs only first, then with the argmin table where S allows
@@ -2022,7 +2129,7 @@ int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_c
         pl->dry_lds_per_cu = (size_t)lds_per_cu;
         int rc;
         try {
-            rc = create(n, p, pl, attempt == 1);
+            rc = create(n, p, pl, attempt == 1, nullptr);   // (initial costs change no address)
             if (rc == GDP_OK) rc = audit(pl, p);
         } catch (const std::bad_alloc &) {
             rc = fail(GDP_E_NOMEM, "host allocation failed");
@@ -2047,19 +2154,13 @@ void gdp_cache_trim(void)
     lane_trim();
 }
 
-int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
+// The parts of gdp_solve_batch.  f0_live: per problem, whether its initial costs are to be uploaded.
+// scan_f0_late: the initial costs have not been looked at yet -- the batch is one part, and they are looked
+// through while the device works on it; *f0_found says afterwards whether any hold more than zeros (or are
+// refused: then the return code says so), in which case nothing has been written to the results.
+static int solve_parts(int32_t n, const gdp_problem *const *p, gdp_result *const *r, size_t budget, std::vector<char> &f0_live,
+                       bool scan_f0_late, bool *f0_found)
 {
-    gdp_clear_error();
-    if (!r) return fail(GDP_E_BADARG, "null results");
-    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
-    for (int i = 0; i < n; ++i) {  // all of them first: nothing is written when one is rejected
-        int rc = validate(p[i], i);
-        if (rc != GDP_OK) return rc;
-    }
-    // A batch whose cost buffers would take more than GALVATRON_DP_ARENA_MB (default 8192) of device
-    // memory is solved in consecutive parts that reuse one allocation: the time to obtain device
-    // memory grows with its size, the time to solve a part does not grow faster than its share.
-    const size_t budget = std::max<size_t>(env_mb("GALVATRON_DP_ARENA_MB", 8192), (size_t)1 << 20);
     int begin = 0, prev_begin = 0;
     gdp_plan *prev = nullptr;
     while (begin < n) {
@@ -2075,7 +2176,7 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
         // (on a stream of its own), while the previous part still runs; it is launched as soon as that
         // one has finished, before that one's results are handed out.
         gdp_plan *pl = nullptr;
-        int rc = create_checked(end - begin, p + begin, &pl);
+        int rc = create_checked(end - begin, p + begin, f0_live.data() + begin, &pl);
         int rp = prev ? run_finish(prev, 0, nullptr) : GDP_OK;
         if (rc == GDP_OK && rp == GDP_OK) {
             pl->one_shot = true;
@@ -2100,10 +2201,56 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
         prev_begin = begin;
         begin = end;
     }
+    int rs = GDP_OK;
+    if (scan_f0_late) {
+        rs = validate_f0_all(n, p, f0_live);
+        for (char c : f0_live) *f0_found = *f0_found || c != 0;
+    }
     int rc = run_finish(prev, 0, nullptr);
-    if (rc == GDP_OK) rc = fetch(prev, r + prev_begin);
+    if (rs != GDP_OK) rc = rs;
+    if (rc == GDP_OK && !*f0_found) rc = fetch(prev, r + prev_begin);
     destroy(prev);
     return rc;
+}
+
+int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r)
+{
+    gdp_clear_error();
+    if (!r) return fail(GDP_E_BADARG, "null results");
+    if (n < 1 || !p) return fail(GDP_E_BADARG, "need at least one problem");
+    bool any_f0 = false;
+    for (int i = 0; i < n; ++i) {  // all of them first: nothing is written when one is rejected
+        const int rc = gdp_validate(p[i], i);
+        if (rc != GDP_OK) return rc;
+        any_f0 = any_f0 || p[i]->f0 != nullptr;
+    }
+    // A batch whose cost buffers would take more than GALVATRON_DP_ARENA_MB (default 8192) of device
+    // memory is solved in consecutive parts that reuse one allocation: the time to obtain device
+    // memory grows with its size, the time to solve a part does not grow faster than its share.
+    const size_t budget = std::max<size_t>(env_mb("GALVATRON_DP_ARENA_MB", 8192), (size_t)1 << 20);
+    try {
+        std::vector<char> f0_live((size_t)n, 0);
+        // Initial costs (gdp_problem.f0) are zeros in every call the reference's own code makes, and looking
+        // through V x S doubles takes as long as solving a small instance.  A batch of one part is therefore
+        // started as if they were zeros and the arrays are looked through while the device works; should one
+        // of them hold anything else, that solve is dropped and the batch solved again with them.
+        size_t bytes = 0;
+        for (int i = 0; i < n && bytes <= budget; ++i) bytes += footprint(p[i]);
+        const bool late = any_f0 && n <= 65535 && bytes <= budget;
+        if (any_f0 && !late) {
+            const int rc = validate_f0_all(n, p, f0_live);
+            if (rc != GDP_OK) return rc;
+        }
+        bool f0_found = false;
+        int rc = solve_parts(n, p, r, budget, f0_live, late, &f0_found);
+        if (rc == GDP_OK && f0_found) {
+            f0_found = false;
+            rc = solve_parts(n, p, r, budget, f0_live, false, &f0_found);
+        }
+        return rc;
+    } catch (const std::bad_alloc &) {
+        return fail(GDP_E_NOMEM, "host allocation failed");
+    }
 }
 
 int gdp_solve(const gdp_problem *p, gdp_result *r)

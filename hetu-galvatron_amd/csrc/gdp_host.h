@@ -11,8 +11,12 @@ int gdp_fail(int code, const char *msg);             // returns code
 int gdp_fail_hip(hipError_t e, const char *what);    // GDP_E_NOMEM for an allocation failure, else GDP_E_HIP
 
 // Host-side checks of one problem (instance number i is for the message only): sizes, null pointers,
-// mem >= 1, other_mem >= 0, inter_index in range, no NaN / -inf, no possible overflow.  Allocates nothing.
+// mem >= 0, other_mem >= 0, inter_index in range, no NaN / -inf, no possible overflow -- everything but the
+// initial costs.  Allocates nothing.
 int gdp_validate(const gdp_problem *p, int i);
+// ... and of its initial costs (gdp_problem.f0; GDP_OK when there are none): no NaN / -inf / -0.0, no possible
+// overflow.  *f0_live (may be null): they hold something other than zeros.  Allocates nothing.
+int gdp_validate_f0(const gdp_problem *p, int i, bool *f0_live);
 
 // Index into GDP_VARIANTS of the register tile ts x r, or -1.
 int gdp_find_variant(int ts, int r);

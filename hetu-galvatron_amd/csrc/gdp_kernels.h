@@ -210,7 +210,10 @@ hipError_t gdp_launch_zero(int32_t *p, int64_t n, hipStream_t stream);
 // buffer alone) this pass recomputes the mem == 0 columns, one lane per bin, in ascending strategy
 // order: candidates from lower strategies come from the buffer the layer writes, the others from the
 // buffer it reads.  One launch per layer only (plans with such strategies never fuse layers).
-hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, int n_inst, int max_V, int layer, hipStream_t stream);
+// lay: the table of n_inst x max_L layer records that belongs to `insts` (the pass keeps to each layer's band
+// of tile_rows-row tiles).
+hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, const GdpDevLayer *lay, int max_L, int tile_rows,
+                                int n_inst, int max_V, int layer, hipStream_t stream);
 // argmin over the last layer's row + backtrack, one wavefront per key (marks: through the stored
 // argmin table; otherwise recomputed from the cost buffers of all layers).
 hipError_t gdp_launch_epilogue(bool marks, const GdpDevInst *insts, const GdpDevKey *keys, int n_key, GdpDevOut *out,

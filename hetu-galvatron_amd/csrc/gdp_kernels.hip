@@ -1122,13 +1122,16 @@ __global__ __launch_bounds__(256) void gdp_init_kernel(const GdpDevInst *__restr
 }
 
 // ---- strategies with a memory cost of 0 -------------------------------------------------------------
-// See gdp_launch_zero_pass.  grid = (blocks of 256 bins, instances).  A lane owns bin v and walks the
+// See gdp_launch_zero_pass.  grid = (blocks of 256 bins, instances).  Only the bins of the layer's band are
+// redone: below it every candidate is +inf (the cells hold +inf, argmin 0, from the fills), above it nothing
+// was written by the layer's launch and nothing is read later.  A lane owns bin v and walks the
 // layer's mem == 0 strategies in ascending order; what it stores for one of them is what it (and only
 // it) reads back as a candidate of the next ones.  Candidates, association and tie-break are the
 // reference's: (f + inter) + intra, ascending source strategies, replaced on strict '<'
 // (csrc/dp_core.cpp:65-72).
 template <bool MARKS>
-__global__ __launch_bounds__(256) void gdp_zero_pass_kernel(const GdpDevInst *insts, int layer)
+__global__ __launch_bounds__(256) void gdp_zero_pass_kernel(const GdpDevInst *insts, const GdpDevLayer *lay, int max_L,
+                                                            int tile_rows, int layer)
 {
     const GdpDevInst *I = insts + blockIdx.y;
     const int32_t *zc = uload(&I->zcols);
@@ -1138,6 +1141,9 @@ __global__ __launch_bounds__(256) void gdp_zero_pass_kernel(const GdpDevInst *in
     const int nz = uload(z);
     const int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (nz == 0 || v >= V) return;
+    const GdpDevLayer *Y = lay + ((int64_t)blockIdx.y * max_L + layer);
+    const int lo = uload(&Y->lo), hi = uload(&Y->hi);
+    if (hi < lo || v < (int64_t)lo * tile_rows || v >= (int64_t)(hi + 1) * tile_rows) return;
     const int rows = uload(&I->SU) + GDP_SRC_PAD, SP = uload(&I->SP), nbuf = uload(&I->nbuf);
     const int64_t hstride = uload(&I->hstride);
     double *H = uload(&I->H);
@@ -1611,14 +1617,15 @@ hipError_t gdp_launch_init(const GdpDevInst *insts, int n_inst, int64_t max_ld, 
     return hipGetLastError();
 }
 
-hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, int n_inst, int max_V, int layer, hipStream_t stream)
+hipError_t gdp_launch_zero_pass(bool marks, const GdpDevInst *insts, const GdpDevLayer *lay, int max_L, int tile_rows,
+                                int n_inst, int max_V, int layer, hipStream_t stream)
 {
     if (n_inst <= 0 || max_V <= 0) return hipSuccess;
     dim3 grid((unsigned)((max_V + 255) / 256), (unsigned)n_inst), block(256);
     if (marks)
-        hipLaunchKernelGGL(gdp_zero_pass_kernel<true>, grid, block, 0, stream, insts, layer);
+        hipLaunchKernelGGL(gdp_zero_pass_kernel<true>, grid, block, 0, stream, insts, lay, max_L, tile_rows, layer);
     else
-        hipLaunchKernelGGL(gdp_zero_pass_kernel<false>, grid, block, 0, stream, insts, layer);
+        hipLaunchKernelGGL(gdp_zero_pass_kernel<false>, grid, block, 0, stream, insts, lay, max_L, tile_rows, layer);
     return hipGetLastError();
 }
 

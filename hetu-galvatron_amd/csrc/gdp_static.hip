@@ -2,9 +2,10 @@
 //
 // Every other compute entry point of the library gets device memory for its cost buffers, argmin
 // table, layer records and results (hipMalloc, or an allocation kept from an earlier plan), a stream,
-// events and page-locked host memory.  Some callers may do none of that: code that runs while a HIP
-// graph is being captured elsewhere in the process, tight serving loops that must not touch the
-// allocator, harnesses that forbid it.  For them this entry point keeps all of its device-side working
+// events and page-locked host memory.  Some callers may do none of that: tight serving loops that must
+// not touch the allocator, harnesses that forbid it.  (It is no call for a process in which a stream is
+// being captured in the global capture mode: synchronous copies and null-stream launches are prohibited
+// then.)  For them this entry point keeps all of its device-side working
 // memory in ONE file-scope device array of GDP_STATIC_SCRATCH_BYTES, builds the device layout of the
 // inputs in a fixed host array, runs on the null stream with synchronous copies, and calls no
 // hipMalloc / hipFree / hipHostMalloc / stream or event creation and no host allocator.
@@ -208,7 +209,9 @@ extern "C" int gdp_solve_static(const gdp_problem *p, gdp_result *r)
 {
     gdp_clear_error();
     if (!p || !r) return gdp_fail(GDP_E_BADARG, "null problem or result");
-    const int rc = gdp_validate(p, 0);
+    bool f0_live = false;
+    int rc = gdp_validate(p, 0);
+    if (rc == GDP_OK) rc = gdp_validate_f0(p, 0, &f0_live);
     if (rc != GDP_OK) return rc;
     if (p->flags & (GDP_EXPORT_F | GDP_EXPORT_MARK))
         return gdp_fail(GDP_E_BADARG, "gdp_solve_static does not export f / mark");
@@ -238,9 +241,24 @@ extern "C" int gdp_solve_static(const gdp_problem *p, gdp_result *r)
     // +inf pads and +inf row of both cost buffers, zeros in the first one (the caller's initial f): whatever
     // the last call left there is overwritten before anything reads it
     e = gdp_launch_init(d_inst, 1, y.ld, y.S, d_lay, y.L, 64, GDP_INIT_PADS | GDP_INIT_ZERO, stream);
+    if (e == hipSuccess && f0_live) {
+        // The caller's initial costs [V][S] into buffer 0, one row per strategy: turned round in the host
+        // array a slice of budget rows at a time (the tables it held are on the device by now; the copies
+        // are synchronous and follow the launch above in stream order).
+        double *stage = reinterpret_cast<double *>(g_stage);
+        double *h0 = reinterpret_cast<double *>(base + y.off_H) + y.P;
+        const int slice = (int)std::max<size_t>(1, STAGE_BYTES / (sizeof(double) * (size_t)y.S));
+        for (int v0 = 0; v0 < y.V && e == hipSuccess; v0 += slice) {
+            const int nv = std::min(slice, y.V - v0);
+            for (int v = 0; v < nv; ++v)
+                for (int s = 0; s < y.S; ++s) stage[(size_t)s * nv + v] = p->f0[(size_t)(v0 + v) * y.S + s];
+            e = hipMemcpy2D(h0 + v0, sizeof(double) * (size_t)y.ld, stage, sizeof(double) * (size_t)nv,
+                            sizeof(double) * (size_t)nv, (size_t)y.S, hipMemcpyHostToDevice);
+        }
+    }
     for (int l = 0; l < y.L && e == hipSuccess; ++l) {
         e = gdp_launch_relax(y.variant, true, 0, d_lay, y.L, 1, y.ntile, y.SP, l, stream);
-        if (e == hipSuccess && y.has_zero) e = gdp_launch_zero_pass(true, d_inst, 1, y.V, l, stream);
+        if (e == hipSuccess && y.has_zero) e = gdp_launch_zero_pass(true, d_inst, d_lay, y.L, 64, 1, y.V, l, stream);
     }
     if (e == hipSuccess)
         e = gdp_launch_epilogue(true, d_inst, reinterpret_cast<const GdpDevKey *>(base + y.off_keys), y.n_key,

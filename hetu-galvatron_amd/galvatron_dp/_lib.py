@@ -61,7 +61,7 @@ class gdp_problem(ctypes.Structure):
     _fields_ = [("L", ctypes.c_int32), ("V", ctypes.c_int32), ("S", ctypes.c_int32),
                 ("mem", _ptr), ("intra", _ptr), ("inter", _ptr), ("inter_index", _ptr),
                 ("n_inter", ctypes.c_int32), ("n_key", ctypes.c_int32),
-                ("other_mem", _ptr), ("other_time", _ptr), ("flags", ctypes.c_uint32)]
+                ("other_mem", _ptr), ("other_time", _ptr), ("flags", ctypes.c_uint32), ("f0", _ptr)]
 
 
 class gdp_result(ctypes.Structure):
@@ -161,7 +161,7 @@ class Problem:
 
     def __init__(self, mem, intra, inter, V: int, other_mem: Sequence[int], other_time: Sequence[float], *,
                  inter_index=None, export_f: bool = False, export_mark: bool = False, launch: str | None = None,
-                 compute_all: bool = False, keep_marks: bool = False):
+                 compute_all: bool = False, keep_marks: bool = False, f0=None):
         self.mem = np.ascontiguousarray(mem, dtype=np.int32)
         if self.mem.ndim != 2:
             raise ValueError("mem must be [L,S]")
@@ -186,6 +186,12 @@ class Problem:
         if self.other_mem.shape != self.other_time.shape:
             raise ValueError("other_mem and other_time must have one entry per key")
         self.n_key = int(self.other_mem.shape[0])
+        # initial costs [V,S] (what the reference's caller leaves in ``_f``); the library treats zeros as None
+        self.f0 = None
+        if f0 is not None:
+            self.f0 = np.ascontiguousarray(f0, dtype=np.float64)
+            if self.f0.size != self.V * self.S:
+                raise ValueError("f0 must be [V,S]")
         if launch not in (None, "fused", "per_layer"):
             raise ValueError("launch must be None, 'fused' or 'per_layer'")
         self.flags = ((GDP_EXPORT_F if export_f else 0) | (GDP_EXPORT_MARK if export_mark else 0) |
@@ -206,7 +212,8 @@ class Problem:
         addr = _addr
         self._c_problem = gdp_problem(
             self.L, self.V, self.S, addr(self.mem), addr(self.intra), addr(self.inter), addr(self.inter_index),
-            int(self.inter.shape[0]), self.n_key, addr(self.other_mem), addr(self.other_time), self.flags)
+            int(self.inter.shape[0]), self.n_key, addr(self.other_mem), addr(self.other_time), self.flags,
+            addr(self.f0))
         self._c_result = gdp_result(addr(self.total), addr(self.remaining), addr(self.res), addr(self.f_out),
                                     addr(self.mark_out))
 

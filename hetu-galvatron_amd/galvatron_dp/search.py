@@ -404,41 +404,44 @@ class SearchEngine:
         if part:
             from concurrent.futures import ThreadPoolExecutor
             pool = ThreadPoolExecutor(1)
-        for task in self.tasks():
-            bsz, chunk, min_tp, max_tp, vsp, embed_sdp = task
-            for sp_search in sp_searches:
-                if (sp_search == 1 and vsp == 1) or (sp_search == 2 and vsp == 0):
-                    continue
-                picked = self._task_strategies(bsz, chunk, min_tp, max_tp, sp_search)
-                if picked is None:
-                    continue
-                cand, mbsz, stage = picked
-                model = self._dp_on_model(cand, stage)
-                model.row_cache = row_cache
-                check_optimal_chunks(self.args.gpu_num, cand, self.optimal_chunk_func, bsz, mbsz, min_tp)
-                ticket, dps = model.fit_begin(bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, mbsz_dict=mbsz)
-                pending.append((task, sp_search, model, ticket, len(all_dps), len(dps), stage))
-                all_dps += dps
-                if pool is not None and len(all_dps) - sent >= part:
-                    solved.append(pool.submit(DPAlg.fit_many, all_dps[sent:]))
-                    sent = len(all_dps)
-        self.solved_instances = len(all_dps)
-        if pool is not None:
-            try:
+        try:
+            for task in self.tasks():
+                bsz, chunk, min_tp, max_tp, vsp, embed_sdp = task
+                for sp_search in sp_searches:
+                    if (sp_search == 1 and vsp == 1) or (sp_search == 2 and vsp == 0):
+                        continue
+                    picked = self._task_strategies(bsz, chunk, min_tp, max_tp, sp_search)
+                    if picked is None:
+                        continue
+                    cand, mbsz, stage = picked
+                    model = self._dp_on_model(cand, stage)
+                    model.row_cache = row_cache
+                    check_optimal_chunks(self.args.gpu_num, cand, self.optimal_chunk_func, bsz, mbsz, min_tp)
+                    ticket, dps = model.fit_begin(bsz, min_tp, max_tp, vsp, embed_sdp, sp_search, mbsz_dict=mbsz)
+                    pending.append((task, sp_search, model, ticket, len(all_dps), len(dps), stage))
+                    all_dps += dps
+                    if pool is not None and len(all_dps) - sent >= part:
+                        solved.append(pool.submit(DPAlg.fit_many, all_dps[sent:]))
+                        sent = len(all_dps)
+            self.solved_instances = len(all_dps)
+            if pool is not None:
                 if sent < len(all_dps):
                     solved.append(pool.submit(DPAlg.fit_many, all_dps[sent:]))
                 fits = []
                 for f in solved:
                     fits += f.result()
-            finally:
-                pool.shutdown(wait=True)
-        elif one_batch:
-            fits = DPAlg.fit_many(all_dps)
-        else:
-            fits = []
-            for _, _, _, _, first, count, _ in pending:
-                fits += DPAlg.fit_many(all_dps[first:first + count])
-        self.strategies = strategies_backup
+            elif one_batch:
+                fits = DPAlg.fit_many(all_dps)
+            else:
+                fits = []
+                for _, _, _, _, first, count, _ in pending:
+                    fits += DPAlg.fit_many(all_dps[first:first + count])
+        finally:
+            # whatever happened while the tasks were prepared or solved: no worker is left solving on the
+            # device, and the engine holds its own strategy list again
+            if pool is not None:
+                pool.shutdown(wait=True, cancel_futures=True)
+            self.strategies = strategies_backup
         if not self.keep_device_cache:
             # the library keeps the device allocations of finished batches for the next one; a search is
             # usually the last thing its process asks of the device, so they are handed back here

@@ -31,6 +31,7 @@ class Instance:
     other_time: dict = field(default_factory=dict)
     inter_tables: np.ndarray | None = None   # f64 [T,S,S] when layers share matrices
     inter_index: np.ndarray | None = None    # int32 [L] into inter_tables
+    f0: np.ndarray | None = None             # f64 [V,S] contents of ``_f`` on entry (None: zeros, as DPAlg passes)
 
     @property
     def L(self) -> int:
@@ -53,6 +54,8 @@ class Instance:
         for k in sorted(self.other_mem):
             h.update(np.array([k, self.other_mem[k]], dtype=np.int64).tobytes())
             h.update(np.array([self.other_time[k]], dtype=np.float64).tobytes())
+        if self.f0 is not None:
+            h.update(np.ascontiguousarray(self.f0, dtype=np.float64).tobytes())
         return h.hexdigest()
 
 
@@ -190,6 +193,18 @@ def galvatron_like() -> Instance:
 
 
 CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4}
+
+
+def with_initial_costs(inst: Instance, rng, *, integer: bool = False, inf_frac: float = 0.0) -> Instance:
+    """``inst`` with a non-zero ``_f`` on entry: the reference relaxes in place from whatever the caller's
+    array holds (csrc/dp_core.cpp:46-47,67).  Finite entries (small integers with ``integer``, so that
+    they tie with the costs), a share ``inf_frac`` of +inf."""
+    V, S = inst.V, inst.S
+    f0 = rng.integers(0, 5, size=(V, S)).astype(np.float64) if integer else rng.uniform(-3.0, 25.0, size=(V, S))
+    if inf_frac > 0:
+        f0 = np.where(rng.uniform(size=(V, S)) < inf_frac, np.inf, f0)
+    inst.f0 = np.ascontiguousarray(f0)
+    return inst
 
 
 def random_instance(rng, L: int, S: int, V: int, *, mem_lo=1, mem_hi=None, integer_costs=False,

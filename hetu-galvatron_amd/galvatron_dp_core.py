@@ -7,12 +7,16 @@
 ``sys.path`` ahead of the reference's ``build/lib`` makes that call run on the MI355X through
 libgalvatron_dp_hip.so; nothing else in the caller changes.
 
+``_f`` is read as the reference reads it: the relaxation starts from whatever the array holds on entry
+(csrc/dp_core.cpp:46-47,67; ``DPAlg`` hands in zeros, dynamic_programming.py:16), ``None`` standing for
+zeros.
+
 Differences from the compiled reference module, all on arguments no caller reads back:
 ``_mark`` and ``_f`` are filled only after ``set_export(True)`` (the argmin table lives on the
 device in a compact form, and copying L*V*S int32 back per call would dominate the run time).
 Inputs on which the reference's result depends on evaluation order or is undefined raise
-``ValueError`` instead of computing something: NaN / -inf costs, negative memory costs, a negative
-``other_mem_cost`` (start row above the table).  A memory cost of 0 is computed with the reference's
+``ValueError`` instead of computing something: NaN / -inf costs (also in ``_f``), a -0.0 in ``_f``,
+negative memory costs, a negative ``other_mem_cost`` (start row above the table).  A memory cost of 0 is computed with the reference's
 in-place order (csrc/dp_core.cpp:58-73).
 """
 from __future__ import annotations
@@ -51,7 +55,7 @@ class SharedInter:
         return self.dense()[item]
 
 
-def _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, other_mem_cost, other_time_cost,
+def _problem(layer_num, max_mem, strategy_num, v_data, _f, inter_cost, intra_cost, other_mem_cost, other_time_cost,
              export):
     L, V, S = int(layer_num), int(max_mem), int(strategy_num)
     mem = np.ascontiguousarray(v_data, dtype=np.int32).reshape(L, S)
@@ -61,9 +65,10 @@ def _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, o
     ot = [float(other_time_cost[k]) if k in other_time_cost else 0.0 for k in keys]  # map::operator[] default
     if isinstance(inter_cost, SharedInter):
         return keys, _lib.Problem(mem, intra, inter_cost.tables.reshape(-1, S, S), V, om, ot,
-                                  inter_index=inter_cost.index.reshape(L), export_f=export, export_mark=export)
+                                  inter_index=inter_cost.index.reshape(L), export_f=export, export_mark=export,
+                                  f0=_f)
     inter = np.ascontiguousarray(inter_cost, dtype=np.float64).reshape(L, S, S)
-    return keys, _lib.Problem(mem, intra, inter, V, om, ot, export_f=export, export_mark=export)
+    return keys, _lib.Problem(mem, intra, inter, V, om, ot, export_f=export, export_mark=export, f0=_f)
 
 
 def _finish(keys, prob, _mark, _f, res_list, export):
@@ -84,7 +89,7 @@ def dynamic_programming_core(layer_num, max_mem, strategy_num, v_data, _mark, _f
     """Same signature and return value as the reference (csrc/dp_core.cpp:24-35,119):
     ``(total_cost: dict key->float, remaining_mem: dict key->int)``; ``res_list[key]`` (int32 [L],
     pre-filled with -1 by the caller) is written in place for feasible keys."""
-    keys, prob = _problem(layer_num, max_mem, strategy_num, v_data, inter_cost, intra_cost, other_mem_cost,
+    keys, prob = _problem(layer_num, max_mem, strategy_num, v_data, _f, inter_cost, intra_cost, other_mem_cost,
                           other_time_cost, _export)
     _lib.solve_batch([prob])
     return _finish(keys, prob, _mark, _f, res_list, _export)
@@ -93,6 +98,6 @@ def dynamic_programming_core(layer_num, max_mem, strategy_num, v_data, _mark, _f
 def dynamic_programming_core_batch(calls):
     """Many reference calls in one device batch.  ``calls`` is a sequence of 11-tuples with the
     positional arguments of ``dynamic_programming_core``; returns the list of its return values."""
-    built = [_problem(c[0], c[1], c[2], c[3], c[6], c[7], c[8], c[9], _export) for c in calls]
+    built = [_problem(c[0], c[1], c[2], c[3], c[5], c[6], c[7], c[8], c[9], _export) for c in calls]
     _lib.solve_batch([b[1] for b in built])
     return [_finish(keys, prob, c[4], c[5], c[10], _export) for (keys, prob), c in zip(built, calls)]

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define GDP_VERSION 101 /* major*10000 + minor*100 + patch */
+#define GDP_VERSION 102 /* major*10000 + minor*100 + patch */
 
 /* return codes */
 #define GDP_OK 0
@@ -63,7 +63,9 @@ extern "C" {
  *   L <- layer_num, V <- max_mem (number of budget bins, valid v in [0,V)),
  *   S <- strategy_num, mem <- v_data, intra <- intra_cost, inter <- inter_cost,
  *   other_mem/other_time <- other_mem_cost/other_time_cost values, in the caller's key order
- *   (the dictionary keys themselves are never used by the arithmetic).              */
+ *   (the dictionary keys themselves are never used by the arithmetic),
+ *   f0 <- the contents of _f on entry: the reference relaxes in place, starting from whatever the
+ *   caller's array holds (csrc/dp_core.cpp:46-47,67; DPAlg hands in zeros, dynamic_programming.py:16). */
 typedef struct gdp_problem {
     int32_t L, V, S;
     const int32_t *mem;         /* [L][S]  memory cost in bins, >= 0.  An entry of 0 is computed with the reference's
@@ -79,6 +81,12 @@ typedef struct gdp_problem {
                                             an entry above V-1 is an infeasible key: total +inf, remaining -1) */
     const double *other_time;   /* [n_key]                                                         */
     uint32_t flags;
+    const double *f0;           /* [V][S] initial costs, or NULL for all zeros.  Entries may be finite or +inf;
+                                            NaN and -inf are refused like in the cost arrays (GDP_E_NONFINITE), and
+                                            so is -0.0 (GDP_E_BADARG): the reference keeps the first of two equal
+                                            candidates, so with a negative zero among them the sign of a zero cost
+                                            would depend on the order of evaluation.  An array of zeros is treated
+                                            as NULL.                                                          */
 } gdp_problem;
 
 /* Outputs of one instance <- reference return values / written arguments (csrc/dp_core.cpp:78-119):
@@ -128,8 +136,9 @@ int gdp_solve(const gdp_problem *p, gdp_result *r);
 int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r);
 
 /* gdp_solve for callers that cannot allocate.  No counterpart in the reference: it exists for callers that
- * may not obtain memory while they run -- code executing while a HIP graph is being captured, serving
- * loops that must stay off the allocator, harnesses that forbid hipMalloc.  Same arguments (host
+ * may not obtain memory while they run -- serving loops that must stay off the allocator, harnesses that
+ * forbid hipMalloc.  (Not for use while a stream is being captured in hipStreamCaptureModeGlobal: the call
+ * makes synchronous copies and launches on the null stream, both prohibited then.)  Same arguments (host
  * pointers, borrowed for the call) and the same results, bit for bit, as gdp_solve, but the call
  * obtains no device memory, no page-locked memory, no stream and no event, and uses no host allocator:
  * its cost buffers, argmin table, tables and results live in one static device array of
@@ -143,7 +152,9 @@ int gdp_solve_batch(int32_t n, const gdp_problem *const *p, gdp_result *const *r
  *   - All calls of a process share the array of their device, which keeps what the last call left; a
  *     call rewrites everything it reads, and calls take a process-wide lock, so they run one after the
  *     other.  Work that other code queues on the null stream is ordered with it as usual. */
-#define GDP_STATIC_SCRATCH_BYTES (64 << 20)
+#ifndef GDP_STATIC_SCRATCH_BYTES
+#define GDP_STATIC_SCRATCH_BYTES (64 << 20) /* held on every device the library runs on, by every process that loads it */
+#endif
 int gdp_solve_static(const gdp_problem *p, gdp_result *r);
 
 /* The same in three steps, so that a caller (or a benchmark) can keep inputs resident in

@@ -120,14 +120,16 @@ def ref_module():
     return _ref
 
 
-def ref_solve(mem, intra, inter, V, other_mem, other_time, *, keep=False):
+def ref_solve(mem, intra, inter, V, other_mem, other_time, *, f0=None, keep=False):
     """Call the reference's compiled ``dynamic_programming_core`` exactly as
-    ``DPAlg.fit`` does (dynamic_programming.py:78-92)."""
+    ``DPAlg.fit`` does (dynamic_programming.py:78-92).  ``f0``: what ``_f`` holds on entry
+    (the reference relaxes in place from it, csrc/dp_core.cpp:46-47,67); None for DPAlg's zeros."""
     mem = np.ascontiguousarray(mem, dtype=np.int32)
     intra = np.ascontiguousarray(intra, dtype=np.float64)
     inter = np.ascontiguousarray(inter, dtype=np.float64)
     L, S = mem.shape
-    f = np.full((V, S), 0, dtype=np.float64)
+    f = np.full((V, S), 0, dtype=np.float64) if f0 is None else np.array(f0, dtype=np.float64, order="C")
+    assert f.shape == (V, S)
     mark = np.full((L, V, S), -1, dtype=np.int32)
     res = {k: np.full(L, -1, dtype=np.int32) for k in other_mem}
     total, rem = ref_module().dynamic_programming_core(L, V, S, mem, mark, f, inter, intra,

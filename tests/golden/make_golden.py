@@ -57,6 +57,11 @@ def cases():
     for i, (L, S, V, hi) in enumerate([(4, 6, 60, 2), (6, 22, 400, 3), (5, 44, 900, 1), (8, 64, 700, 4), (3, 65, 300, 2),
                                        (7, 9, 513, 0), (10, 40, 2000, 6), (2, 88, 640, 1)]):
         c[f"zeromem_{i}"] = ("zeromem", {"seed": 4000 + i, "L": L, "S": S, "V": V, "mem_hi": hi})
+    # a non-zero ``_f`` on entry: the relaxation starts from it (csrc/dp_core.cpp:46-47,67)
+    for i, (L, S, V, zero_mem) in enumerate([(3, 5, 200, False), (6, 22, 900, False), (5, 44, 1500, False), (4, 64, 2048, False),
+                                             (7, 40, 3000, False), (3, 88, 700, False), (5, 22, 600, True), (4, 65, 500, True)]):
+        c[f"initf_{i}"] = ("initial_f", {"seed": 5000 + i, "L": L, "S": S, "V": V, "zero_mem": zero_mem})
+    c["initf_galvatron_like"] = ("initial_f_galvatron_like", {})
     return c
 
 
@@ -95,6 +100,14 @@ def build_case(builder: str, kw: dict) -> W.Instance:
             big = rng.uniform(size=inst.mem.shape) < 0.3
             inst.mem[big] = rng.integers(1, max(2, kw["V"] // (kw["L"] + 1)), size=int(big.sum()))
         return inst
+    if builder == "initial_f":
+        rng = np.random.Generator(np.random.PCG64(kw["seed"]))
+        inst = W.random_instance(rng, kw["L"], kw["S"], kw["V"], mem_lo=0 if kw["zero_mem"] else 1,
+                                 mem_hi=max(2, kw["V"] // (kw["L"] + 1)), integer_costs=bool(kw["seed"] % 2),
+                                 per_layer_inter=bool(kw["seed"] % 3), inf_frac=0.1 * (kw["seed"] % 4 == 0), n_keys=4)
+        return W.with_initial_costs(inst, rng, integer=bool(kw["seed"] % 2), inf_frac=0.05 * (kw["seed"] % 2 == 0))
+    if builder == "initial_f_galvatron_like":
+        return W.with_initial_costs(W.galvatron_like(), np.random.Generator(np.random.PCG64(78)), inf_frac=0.01)
     if builder == "galvatron_like":
         return W.galvatron_like()
     return getattr(W, builder)(**kw)
@@ -106,7 +119,7 @@ def solve_case(item):
     inst = build_case(builder, kw)
     t0 = time.time()
     total, res, rem, f, mark = O.ref_solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem,
-                                           inst.other_time, keep=True)
+                                           inst.other_time, f0=inst.f0, keep=True)
     dt = time.time() - t0
     keys = sorted(total)
     rec = {

@@ -49,7 +49,7 @@ def hip_solve(inst, export=False):
     (dynamic_programming.py:78-92)."""
     import galvatron_dp_core as shim
     L, S, V = inst.L, inst.S, inst.V
-    f = np.full((V, S), 0, dtype=np.float64)
+    f = np.full((V, S), 0, dtype=np.float64) if inst.f0 is None else np.array(inst.f0, dtype=np.float64, order="C")
     mark = np.full((L, V, S), -1, dtype=np.int32) if export else np.zeros((1, 1, 1), dtype=np.int32)
     res = {k: np.full(L, -1, dtype=np.int32) for k in inst.other_mem}
     shim.set_export(export)

@@ -27,8 +27,8 @@ def test_header_symbols_are_exported():
 
 
 def test_version_and_struct_sizes():
-    assert _lib.lib().gdp_version() == 101
-    assert ctypes.sizeof(_lib.gdp_problem) == 80
+    assert _lib.lib().gdp_version() == 102
+    assert ctypes.sizeof(_lib.gdp_problem) == 88
     assert ctypes.sizeof(_lib.gdp_result) == 40
     assert ctypes.sizeof(_lib.gdp_timing) == 64
 
@@ -71,6 +71,19 @@ def test_validation_happens_before_any_device_work():
     assert rc == _lib.GDP_E_BADARG and "other_mem" in msg
     too_tall = _lib.Problem(mem, intra, inter, (1 << 30) + 1, [0], [0.0])
     assert rc_of(too_tall)[0] == _lib.GDP_E_BADARG
+    # the initial costs (what the reference's caller leaves in _f): NaN and -inf like in the cost arrays, and
+    # no negative zero; zeros and +inf are fine (checked with the layout audit, which needs no device)
+    f0 = np.ones((10, 3))
+    for bad_value, code in ((np.nan, _lib.GDP_E_NONFINITE), (-np.inf, _lib.GDP_E_NONFINITE), (-0.0, _lib.GDP_E_BADARG),
+                            (1e300, _lib.GDP_E_NONFINITE)):
+        g = f0.copy(); g[7, 1] = bad_value
+        rc, msg = rc_of(_lib.Problem(mem, intra, inter, 10, [0], [0.0], f0=g))
+        assert rc == code and ("f0" in msg or "overflow" in msg), (bad_value, rc, msg)
+    with pytest.raises(ValueError):
+        _lib.Problem(mem, intra, inter, 10, [0], [0.0], f0=np.ones((9, 3)))
+    ok = f0.copy(); ok[2, 2] = np.inf
+    _lib.check_layout([_lib.Problem(mem, intra, inter, 10, [0], [0.0], f0=ok)])
+    _lib.check_layout([_lib.Problem(mem, intra, inter, 10, [0], [0.0], f0=np.zeros((10, 3)))])
 
 
 def test_static_entry_point_refuses_on_the_host():
@@ -125,3 +138,34 @@ def test_problem_points_at_the_arrays_it_keeps():
     assert list(p.total) == [np.inf, np.inf] and list(p.remaining) == [-1, -1] and (p.res == -1).all()
     q = _lib.Problem(mem.copy(), intra.copy(), inter.copy(), 10, [], [])
     assert q.n_key == 0 and q.total.shape == (0,)
+
+
+def test_static_entry_point_links_against_nothing_that_allocates(tmp_path):
+    """gdp_solve_static exists for callers that may not obtain memory.  Its translation unit is compiled
+    alone and its undefined symbols are looked through: no device, page-locked or host allocator, no stream
+    or event creation; and of the library's other translation units only helpers that allocate nothing
+    (validation, error text, kernel launchers)."""
+    import shutil
+    import subprocess
+    from galvatron_dp import _build
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    if shutil.which(hipcc) is None:
+        pytest.skip("no hipcc")
+    obj = str(tmp_path / "gdp_static.o")
+    flags = [f for f in _build.HIPCC_FLAGS if f != "-shared"]
+    proc = subprocess.run([hipcc] + flags + ["-c", os.path.join(_build.CSRC, "gdp_static.hip"), "-o", obj],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    undefined = subprocess.run(["nm", "-u", "-C", obj], stdout=subprocess.PIPE, text=True, check=True).stdout
+    names = [ln.split(None, 1)[1].strip() for ln in undefined.splitlines() if ln.strip().startswith("U ")]
+    assert any(n.startswith("hipGetSymbolAddress") for n in names), names
+    forbidden = ("hipMalloc", "hipHostMalloc", "hipExtMalloc", "hipHostAlloc", "hipMemAlloc", "hipStreamCreate",
+                 "hipEventCreate", "hipFree", "hipHostFree", "operator new", "operator delete", "malloc", "calloc",
+                 "realloc", "posix_memalign", "aligned_alloc", "std::__throw_length_error", "std::__throw_bad_alloc")
+    for n in names:
+        assert not any(n == f or n.startswith(f + "(") or n.startswith(f + "[") or (f.startswith("hip") and n.startswith(f))
+                       for f in forbidden), f"gdp_static.hip refers to {n}"
+    allowed_own = {"gdp_clear_error", "gdp_fail", "gdp_fail_hip", "gdp_validate", "gdp_validate_f0", "gdp_find_variant",
+                   "gdp_launch_init", "gdp_launch_relax", "gdp_launch_zero_pass", "gdp_launch_epilogue"}
+    own = {n.split("(")[0] for n in names if n.startswith("gdp_")}
+    assert own <= allowed_own, own - allowed_own

@@ -110,6 +110,23 @@ def test_costs_only_and_mark_table_modes_agree(golden, name, launch, keep_marks)
         assert t.relax_bytes == cells * (17 if keep_marks else 16)
 
 
+@pytest.mark.parametrize("keep_marks", [False, True])
+@pytest.mark.parametrize("name", [f"zeromem_{i}" for i in range(8)])
+def test_memory_costs_of_zero_with_rows_skipped_and_unwritten_cells_poisoned(golden, name, keep_marks):
+    """The pass that redoes the strategies with a memory cost of 0 keeps to the layer's band: rows above
+    it were never written by the layer's launch (they read as NaN here), rows below it hold their fill."""
+    rec = golden[name]
+    inst = H.build_case(rec)
+    prob = _problem(inst, keep_marks=keep_marks)
+    with _lib.Plan([prob]) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)
+        for run in range(2):
+            t = plan.run(1)
+            plan.fetch()
+            _check_against_golden(prob, rec, f"{name} keep_marks={keep_marks} run {run}")
+    assert t.executed <= t.relaxations
+
+
 def test_batch_solved_in_parts_and_allocation_reuse(golden, monkeypatch):
     """A batch above the device-memory budget of one allocation is solved in consecutive parts; the
     allocation of a finished plan is reused by the next one (stale contents must not matter) and

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 SMALL = ([f"ties_{i}" for i in range(10)] + [f"rand_{i}" for i in range(10)] +
          [f"infeasible_{i}" for i in range(10)] + [f"cfg3_smallV_{i}" for i in range(8)] +
          ["cfg2_small", "cfg4_small", "galvatron_like", "cfg0", "cfg0_other_time"] +
-         [f"zeromem_{i}" for i in range(8)])
+         [f"zeromem_{i}" for i in range(8)] + [f"initf_{i}" for i in range(8)] + ["initf_galvatron_like"])
 
 
 @pytest.mark.parametrize("name", SMALL)
@@ -30,7 +30,8 @@ def test_golden_covers_every_benchmark_config_on_the_gpu_box(golden):
         assert name in golden, name
 
 
-@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4"] + [f"zeromem_{i}" for i in range(8)])
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg4"] + [f"zeromem_{i}" for i in range(8)] +
+                         [f"initf_{i}" for i in range(8)] + ["initf_galvatron_like"])
 def test_golden_full_size(golden, name):
     assert name in golden, f"the committed vectors have no case {name}: a lost fixture is a failure, not a skip"
     rec = golden[name]

@@ -12,7 +12,7 @@ needs_ref = pytest.mark.skipif(not O.ref_available(), reason="oracle/_ref not bu
 CPU_GOLDEN = ([f"ties_{i}" for i in range(10)] + [f"rand_{i}" for i in range(10)] +
               [f"infeasible_{i}" for i in range(10)] + [f"cfg3_smallV_{i}" for i in range(8)] +
               ["cfg2_small", "cfg4_small", "galvatron_like", "cfg0", "cfg0_other_time", "cfg1"] +
-              [f"zeromem_{i}" for i in range(8)])
+              [f"zeromem_{i}" for i in range(8)] + [f"initf_{i}" for i in range(8)] + ["initf_galvatron_like"])
 
 
 @pytest.mark.parametrize("name", CPU_GOLDEN)
@@ -20,7 +20,7 @@ def test_oracle_matches_golden(golden, name):
     rec = golden[name]
     inst = H.build_case(rec)
     total, res, rem, f, mark = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time,
-                                       keep=True)
+                                       f0=inst.f0, keep=True)
     H.assert_same_results((total, res, rem), H.golden_results(rec), name)
     assert H.sha(f) == rec["f_sha256"]
     assert H.sha(mark) == rec["mark_sha256"]
@@ -52,6 +52,22 @@ def test_oracle_vs_reference_build_random(seed):
                              inf_frac=0.15 * (seed % 3 == 0), over_frac=0.1 * (seed % 4 == 0), n_keys=4)
     a = O.solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, keep=True)
     b = O.ref_solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, keep=True)
+    H.assert_same_results(a[:3], b[:3], f"seed {seed}")
+    assert a[3].tobytes() == b[3].tobytes() and np.array_equal(a[4], b[4])
+
+
+@needs_ref
+@pytest.mark.parametrize("seed", range(12))
+def test_oracle_vs_reference_build_with_initial_costs(seed):
+    """``_f`` is read, not only written: the reference relaxes in place from whatever the caller's array
+    holds (csrc/dp_core.cpp:46-47,67).  Random finite / +inf initial costs, memory costs of 0 included."""
+    rng = np.random.Generator(np.random.PCG64(1700 + seed))
+    L, S, V = int(rng.integers(1, 8)), int(rng.integers(1, 70)), int(rng.integers(20, 700))
+    inst = W.random_instance(rng, L, S, V, integer_costs=bool(seed % 2), mem_hi=max(1, V // (L + 1)),
+                             mem_lo=0 if seed % 4 == 0 else 1, inf_frac=0.1 * (seed % 3 == 0), n_keys=4)
+    W.with_initial_costs(inst, rng, integer=bool(seed % 2), inf_frac=0.1 * (seed % 5 == 0))
+    a = O.solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, f0=inst.f0, keep=True)
+    b = O.ref_solve(inst.mem, inst.intra, inst.inter, V, inst.other_mem, inst.other_time, f0=inst.f0, keep=True)
     H.assert_same_results(a[:3], b[:3], f"seed {seed}")
     assert a[3].tobytes() == b[3].tobytes() and np.array_equal(a[4], b[4])
 

@@ -30,11 +30,21 @@ def test_static_entry_point_matches_gdp_solve_twice_in_a_row(golden):
     rng = np.random.Generator(np.random.PCG64(77))
     big = W.random_instance(rng, 12, 44, 9000, mem_hi=900, inf_frac=0.1)
     small = W.random_instance(rng, 5, 22, 1500, integer_costs=True, mem_hi=300, inf_frac=0.05)
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
     for n, inst in enumerate((big, small)):
         want = _problem(inst)
         _lib.solve_batch([want])                       # gdp_solve_batch of one instance is gdp_solve
         got = _problem(inst)
+        before = free_bytes()
         _lib.solve_static(got)
+        assert n == 0 or free_bytes() == before, "the second call changed the free device memory"
         _same(got, want, f"call {n}")
         assert np.isfinite(want.total).any(), "the case should have feasible keys"
 
