@@ -29,7 +29,16 @@ in HBM (``gdp_plan_create`` has run).  Prints ONE JSON line.
                    over the dispatch duration; null where not profiled): the peak assumes 2.4 GHz.
                    ``traffic`` is the measured HBM-side byte count per launch from profiles/, given
                    only while the kernel sources still hash to what was profiled.
-* ``vs_baseline``  null: the reference publishes no number for this path.
+* ``vs_baseline``  null: the reference publishes no number for this path.  ``vs_cpu_baseline_same_run`` is
+                   ``value`` over ``cpu_baseline.value``: the reference's own code on ONE core of this host, timed
+                   in this run -- a measured companion figure, not a published baseline.
+* ``also.sweep_llama_like``  a whole search as the engine runs it (``SearchEngine.parallelism_optimization``,
+                   the counterpart of search_engine.py:339-537, on a synthetic llama-like profile): all DP
+                   instances of all tasks in one device batch.  Wall time of the call, the device's share (HIP
+                   events around the kernels of every part of the batch, summed), the host's share (cost models,
+                   input assembly, layout, copies: the rest), the relaxations of the mixed-shape batch and their
+                   rate against the roofs, and whether the results equal the ones recorded from the reference's
+                   engine (tests/golden/sweep_golden.json).
 * ``also``         the other workloads, shorter legs, each with its own fractions and a ``bit_exact``
                    flag: results compared, outside the timed region, with the committed vectors
                    written from the reference's compiled dp_core (tests/golden/dp_core_golden.json).
@@ -70,11 +79,11 @@ PEAK_HBM_GBS = 8000.0
 # bench line carries it only while both still match, null otherwise.
 MEASURED_TRAFFIC = {
     # workload (+ mode): (bytes per launch, kernel sources hash, register tile "TSxR", profile)
-    "cfg2": (12.131e9, "18eee00e2b9b2749", "16x1", "profiles/gdp_relax_fused_kernel_cfg2.txt"),                 # algorithmic 10.737e9
-    "cfg2+row_skipping": (7.651e9, "18eee00e2b9b2749", "16x1", "profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt"),
-    "cfg2+mark_table": (12.212e9, "18eee00e2b9b2749", "8x2", "profiles/gdp_relax_fused_kernel_cfg2_mark_table.txt"),  # algorithmic 11.409e9
-    "cfg3": (45.84e9, "18eee00e2b9b2749", "15x3", "profiles/gdp_relax_fused_kernel_cfg3.txt"),   # algorithmic 44.3e9; average of the 4 launches of a solve
-    "cfg4": (17.612e9, "18eee00e2b9b2749", "15x3", "profiles/gdp_relax_fused_kernel_cfg4.txt"),                 # algorithmic 17.716e9
+    "cfg2": (12.131e9, "3ef1fc3c77e9bc65", "16x1", "profiles/gdp_relax_fused_kernel_cfg2.txt"),                 # algorithmic 10.737e9
+    "cfg2+row_skipping": (7.651e9, "3ef1fc3c77e9bc65", "16x1", "profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt"),
+    "cfg2+mark_table": (12.212e9, "3ef1fc3c77e9bc65", "8x2", "profiles/gdp_relax_fused_kernel_cfg2_mark_table.txt"),  # algorithmic 11.409e9
+    "cfg3": (45.76e9, "3ef1fc3c77e9bc65", "15x3", "profiles/gdp_relax_fused_kernel_cfg3.txt"),   # algorithmic 44.3e9; average of the 4 launches of a solve
+    "cfg4": (17.606e9, "3ef1fc3c77e9bc65", "15x3", "profiles/gdp_relax_fused_kernel_cfg4.txt"),                 # algorithmic 17.716e9
 }
 KERNEL_SOURCES = ("hetu-galvatron_amd/csrc/gdp_kernels.hip", "hetu-galvatron_amd/csrc/gdp_kernels.h")
 GOLDEN = os.path.join(ROOT, "tests", "golden", "dp_core_golden.json")
@@ -144,6 +153,66 @@ def _problems(workload: str, compute_all: bool = True, keep_marks: bool = False)
     return insts, probs
 
 
+def _host_description():
+    """CPU model and number of logical processors of this host (for the CPU baseline figures)."""
+    model = None
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for ln in fh:
+                if ln.lower().startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "nproc": os.cpu_count()}
+
+
+def _sweep_leg(name: str = "llama_like", repeats: int = 3):
+    """One whole search through ``galvatron_dp.search.SearchEngine`` (scenario ``name`` of tests/sweep_cases.py: a
+    synthetic profile, the argument records handed in); median of ``repeats`` runs after one untimed run."""
+    import tempfile
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import sweep_cases as S
+    from galvatron_dp import _lib, cost_models
+    from galvatron_dp.search import SearchEngine
+    runs = []
+    summary = None
+    for rep in range(repeats + 1):
+        with tempfile.TemporaryDirectory() as wd:
+            eng = S.build(SearchEngine, cost_models, name, wd)
+            eng.keep_device_cache = True                  # as inside a search service: allocations are reused
+            _lib.batch_stats_begin()
+            t0 = time.perf_counter()
+            thr = eng.parallelism_optimization()
+            wall = (time.perf_counter() - t0) * 1e3
+            st = _lib.batch_stats_end()
+            if rep == 0:
+                summary = S.summarize(eng, thr, wd)
+                continue
+            runs.append((wall, st, eng.solved_instances))
+    _lib.cache_trim()
+    runs.sort(key=lambda r: r[0])
+    wall, st, n_inst = runs[len(runs) // 2]
+    bit_exact = None
+    gpath = os.path.join(ROOT, "tests", "golden", "sweep_golden.json")
+    if os.path.exists(gpath):
+        with open(gpath) as fh:
+            ref = json.load(fh)["sweeps"].get(name)
+        if ref is not None:
+            bit_exact = (summary["throughput"] == ref["throughput"] and summary["files"] == ref["files"] and
+                         summary["table"] == ref["table"])
+    dev_s = st.device_ms * 1e-3
+    return {"scenario": name, "dp_instances": int(n_inst), "tasks_results": len(summary["table"]),
+            "search_wall_ms": wall, "device_busy_ms": st.device_ms, "host_ms": wall - st.device_ms,
+            "relaxations": st.relaxations, "relaxations_executed_fraction": st.executed / max(st.relaxations, 1.0),
+            "value_wall": st.relaxations / (wall * 1e-3), "value_device": st.relaxations / max(dev_s, 1e-12),
+            "roofline_frac_valu_fp64_device": 2.0 * st.executed / max(dev_s, 1e-12) / 1e12 / PEAK_FP64_VALU_TFLOPS,
+            "batch_parts": int(st.parts), "parts_by_launch_scheme": {"flow": int(st.flow_parts), "fused": int(st.fused_parts),
+                                                                      "per_layer": int(st.per_layer_parts)},
+            "bit_exact": bit_exact}
+
+
 def _cpu_baseline(workload: str, budget_s: float = 15.0):
     """Reference dp_core (or the C port) on the first layers of the workload's first instance."""
     import numpy as np
@@ -164,7 +233,7 @@ def _cpu_baseline(workload: str, budget_s: float = 15.0):
     fn(mem, intra, inter, inst.V, inst.other_mem, inst.other_time)
     dt = time.perf_counter() - t0
     relax = n_layers * per_layer
-    return {"value": relax / dt, "unit": "relaxations/s", "cores": 1,
+    return {"value": relax / dt, "unit": "relaxations/s", "cores": 1, **_host_description(),
             "kind": "reference" if use_ref else "port",
             "sample": f"first {n_layers} of {inst.L} layers of {inst.name} (V={inst.V}, S={inst.S}), "
                       f"{relax:.3g} relaxations in {dt:.2f} s, single thread, includes the host argmin-table "
@@ -198,7 +267,7 @@ def _cpu_baseline_all_cores(budget_s: float = 8.0):
         t0 = time.perf_counter()
         relax = sum(sum(pool.map(one, insts)) for _ in range(rounds))
         dt = time.perf_counter() - t0
-    return {"value": relax / dt, "unit": "relaxations/s", "cores": cores, "kind": "port",
+    return {"value": relax / dt, "unit": "relaxations/s", "cores": cores, **_host_description(), "kind": "port",
             "sample": f"first {n_layers} layers of {len(insts)} cfg3 instances, {rounds} rounds, one thread per instance, "
                       f"{relax:.3g} relaxations in {dt:.2f} s"}
 
@@ -219,7 +288,8 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true",
                     help="leave out the row-skipping and mark-table legs (profiling runs: the trace then holds the "
                          "headline's launches alone)")
-    ap.add_argument("--also", default="cfg3,cfg0,cfg1,cfg4,galvatron_like", help="comma-separated extra workloads summarised in the same line")
+    ap.add_argument("--also", default="cfg3,cfg0,cfg1,cfg4,galvatron_like,sweep_llama_like",
+                    help="comma-separated extra workloads summarised in the same line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run three device-to-device copies of 1 GiB (a kernel of known traffic, to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run) and exit")
@@ -369,6 +439,9 @@ def main() -> int:
     }
     also = {}
     for w in [x for x in a.also.split(",") if x and x != a.workload]:
+        if w.startswith("sweep_"):
+            also[w] = _sweep_leg(w[len("sweep_"):])
+            continue
         mm = measure(w, max(3, a.steps // 4), 1, host_leg=not a.headline_only, check=True)
         ff = fractions(mm)
         also[w] = {"value": mm["value"], "ms_per_step": mm["ms_per_step"], "instances": len(mm["insts"]),
@@ -402,6 +475,10 @@ def main() -> int:
                                    "bit_exact": mk["bit_exact"]}
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = _cpu_baseline(a.workload)
+        line["vs_cpu_baseline_same_run"] = {
+            "ratio": m["value"] / line["cpu_baseline"]["value"],
+            "meaning": "value / cpu_baseline.value: the same-run figure of the reference's code on one core of this "
+                       "host, not a published baseline (vs_baseline stays null: none is published)"}
         if "cfg3" in also:
             also["cfg3"]["cpu_baseline_all_cores"] = _cpu_baseline_all_cores()
     print(json.dumps(line))

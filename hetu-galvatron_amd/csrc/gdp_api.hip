@@ -352,6 +352,11 @@ void fused_turn_give()
     g_fused_cv.notify_one();
 }
 
+// gdp_batch_stats_begin / _end: what the batches of the process did in between.
+std::mutex g_stats_mu;
+bool g_stats_on = false;
+gdp_batch_stats g_stats = {};
+
 struct HostInst {
     int orig;  // index in the caller's arrays
     int L, V, S, SP, SU, P, ntile, n_key, n_inter, variant, nbuf;
@@ -2148,6 +2153,23 @@ void gdp_debug_shared_device(int32_t seems_shared)
     g_last_give_up_ms.store(seems_shared ? steady_ms() : -1, std::memory_order_relaxed);
 }
 
+void gdp_batch_stats_begin(void)
+{
+    std::lock_guard<std::mutex> lk(g_stats_mu);
+    g_stats = gdp_batch_stats();
+    g_stats_on = true;
+}
+
+int gdp_batch_stats_end(gdp_batch_stats *out)
+{
+    gdp_clear_error();
+    if (!out) return fail(GDP_E_BADARG, "null statistics record");
+    std::lock_guard<std::mutex> lk(g_stats_mu);
+    g_stats_on = false;
+    *out = g_stats;
+    return GDP_OK;
+}
+
 void gdp_cache_trim(void)
 {
     arena_trim(-1);
@@ -2163,6 +2185,26 @@ static int solve_parts(int32_t n, const gdp_problem *const *p, gdp_result *const
 {
     int begin = 0, prev_begin = 0;
     gdp_plan *prev = nullptr;
+    bool stats = false;
+    {
+        std::lock_guard<std::mutex> lk(g_stats_mu);
+        stats = g_stats_on;
+    }
+    const int mode = stats ? 1 : 0;   // events around the kernels of every part
+    auto finish = [&](gdp_plan *pl) {
+        gdp_timing t;
+        const int rc = run_finish(pl, mode, stats ? &t : nullptr);
+        if (rc == GDP_OK && stats) {
+            std::lock_guard<std::mutex> lk(g_stats_mu);
+            g_stats.relaxations += t.relaxations;
+            g_stats.executed += t.executed;
+            g_stats.device_ms += t.total_ms;
+            g_stats.instances += pl->n;
+            g_stats.parts += 1;
+            (t.flow ? g_stats.flow_parts : t.fused ? g_stats.fused_parts : g_stats.per_layer_parts) += 1;
+        }
+        return rc;
+    };
     while (begin < n) {
         int end = begin;
         size_t bytes = 0;
@@ -2177,10 +2219,10 @@ static int solve_parts(int32_t n, const gdp_problem *const *p, gdp_result *const
         // one has finished, before that one's results are handed out.
         gdp_plan *pl = nullptr;
         int rc = create_checked(end - begin, p + begin, f0_live.data() + begin, &pl);
-        int rp = prev ? run_finish(prev, 0, nullptr) : GDP_OK;
+        int rp = prev ? finish(prev) : GDP_OK;
         if (rc == GDP_OK && rp == GDP_OK) {
             pl->one_shot = true;
-            rc = run_enqueue(pl, 0);
+            rc = run_enqueue(pl, mode);
             if (rc != GDP_OK && pl->holds_fused) {
                 (void)hipStreamSynchronize(pl->stream);
                 pl->holds_fused = false;
@@ -2206,7 +2248,7 @@ static int solve_parts(int32_t n, const gdp_problem *const *p, gdp_result *const
         rs = validate_f0_all(n, p, f0_live);
         for (char c : f0_live) *f0_found = *f0_found || c != 0;
     }
-    int rc = run_finish(prev, 0, nullptr);
+    int rc = finish(prev);
     if (rs != GDP_OK) rc = rs;
     if (rc == GDP_OK && !*f0_found) rc = fetch(prev, r + prev_begin);
     destroy(prev);

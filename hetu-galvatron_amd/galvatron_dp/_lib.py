@@ -39,7 +39,8 @@ GDP_STATIC_SCRATCH_BYTES = 64 << 20
 
 EXPORTED_SYMBOLS = ("gdp_solve", "gdp_solve_batch", "gdp_solve_static", "gdp_plan_create", "gdp_plan_run", "gdp_plan_fetch",
                     "gdp_plan_destroy", "gdp_plan_set_option", "gdp_cache_trim", "gdp_last_error", "gdp_version",
-                    "gdp_device_info", "gdp_debug_check_layout", "gdp_debug_shared_device")
+                    "gdp_device_info", "gdp_debug_check_layout", "gdp_debug_shared_device", "gdp_batch_stats_begin",
+                    "gdp_batch_stats_end")
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -74,6 +75,12 @@ class gdp_timing(ctypes.Structure):
                 ("relax_bytes", ctypes.c_double), ("tile_ts", ctypes.c_int32), ("tile_r", ctypes.c_int32),
                 ("keep_marks", ctypes.c_int32), ("chunk", ctypes.c_int32),
                 ("latency_variant", ctypes.c_int32), ("flow", ctypes.c_int32)]
+
+
+class gdp_batch_stats(ctypes.Structure):
+    _fields_ = [("relaxations", ctypes.c_double), ("executed", ctypes.c_double), ("device_ms", ctypes.c_double),
+                ("instances", ctypes.c_int64), ("parts", ctypes.c_int64), ("flow_parts", ctypes.c_int64),
+                ("fused_parts", ctypes.c_int64), ("per_layer_parts", ctypes.c_int64)]
 
 
 _lib = None
@@ -116,6 +123,10 @@ def lib() -> ctypes.CDLL:
         L.gdp_debug_check_layout.restype = ctypes.c_int
         L.gdp_debug_shared_device.argtypes = [ctypes.c_int32]
         L.gdp_debug_shared_device.restype = None
+        L.gdp_batch_stats_begin.argtypes = []
+        L.gdp_batch_stats_begin.restype = None
+        L.gdp_batch_stats_end.argtypes = [ctypes.POINTER(gdp_batch_stats)]
+        L.gdp_batch_stats_end.restype = ctypes.c_int
         _lib = L
     return _lib
 
@@ -253,6 +264,18 @@ def debug_shared_device(seems_shared: bool) -> None:
     """gdp_debug_shared_device: puts the library into (or takes it out of) the state it enters when a waiting
     launch was given up: launches that never wait are then chosen wherever the choice is the library's."""
     lib().gdp_debug_shared_device(1 if seems_shared else 0)
+
+
+def batch_stats_begin() -> None:
+    """gdp_batch_stats_begin: start adding up what the process's gdp_solve_batch calls do."""
+    lib().gdp_batch_stats_begin()
+
+
+def batch_stats_end() -> gdp_batch_stats:
+    """gdp_batch_stats_end: stop, and return the sums (relaxations, device time of the parts, ...)."""
+    s = gdp_batch_stats()
+    _check(lib().gdp_batch_stats_end(ctypes.byref(s)))
+    return s
 
 
 def solve_static(problem: Problem) -> None:

@@ -92,7 +92,7 @@ class DPAlg:
         """The eleven positional arguments of the plugin call for this instance
         (dynamic_programming.py:79-91), with a fresh ``res_list``."""
         res_list = {k: np.full(self.layer_num, -1, dtype=np.int32) for k in self.other_mem_cost}
-        if galvatron_dp_core._export:
+        if galvatron_dp_core.export_enabled():
             self._f = np.full((self.max_mem, self.strategy_num), 0, dtype=np.float64)
             self._mark = np.full((self.layer_num, self.max_mem, self.strategy_num), -1, dtype=np.int32)
         return (self.layer_num, self.max_mem, self.strategy_num, self.v_data, self._mark, self._f, self.inter_cost,

@@ -21,20 +21,27 @@ in-place order (csrc/dp_core.cpp:58-73).
 """
 from __future__ import annotations
 
+import threading
+
 import numpy as np
 
 from galvatron_dp import _lib
 
-__all__ = ["dynamic_programming_core", "dynamic_programming_core_batch", "set_export", "SharedInter"]
+__all__ = ["dynamic_programming_core", "dynamic_programming_core_batch", "set_export", "export_enabled", "SharedInter"]
 
-_export = False
+_state = threading.local()      # per thread: the reference's parallel search calls the plugin from many threads
 
 
 def set_export(flag: bool) -> None:
-    """When true, ``_f`` and ``_mark`` are written exactly as the reference writes them
-    (csrc/dp_core.cpp:61-62,72-73)."""
-    global _export
-    _export = bool(flag)
+    """When true, the calls of THIS thread write ``_f`` and ``_mark`` exactly as the reference writes them
+    (csrc/dp_core.cpp:61-62,72-73).  Other threads are not affected; ``dynamic_programming_core_batch`` also
+    takes the choice per call (``export=``)."""
+    _state.export = bool(flag)
+
+
+def export_enabled() -> bool:
+    """What ``set_export`` last set in the calling thread (False if it never did)."""
+    return getattr(_state, "export", False)
 
 
 class SharedInter:
@@ -89,15 +96,18 @@ def dynamic_programming_core(layer_num, max_mem, strategy_num, v_data, _mark, _f
     """Same signature and return value as the reference (csrc/dp_core.cpp:24-35,119):
     ``(total_cost: dict key->float, remaining_mem: dict key->int)``; ``res_list[key]`` (int32 [L],
     pre-filled with -1 by the caller) is written in place for feasible keys."""
+    export = export_enabled()
     keys, prob = _problem(layer_num, max_mem, strategy_num, v_data, _f, inter_cost, intra_cost, other_mem_cost,
-                          other_time_cost, _export)
+                          other_time_cost, export)
     _lib.solve_batch([prob])
-    return _finish(keys, prob, _mark, _f, res_list, _export)
+    return _finish(keys, prob, _mark, _f, res_list, export)
 
 
-def dynamic_programming_core_batch(calls):
+def dynamic_programming_core_batch(calls, export=None):
     """Many reference calls in one device batch.  ``calls`` is a sequence of 11-tuples with the
-    positional arguments of ``dynamic_programming_core``; returns the list of its return values."""
-    built = [_problem(c[0], c[1], c[2], c[3], c[5], c[6], c[7], c[8], c[9], _export) for c in calls]
+    positional arguments of ``dynamic_programming_core``; returns the list of its return values.
+    ``export``: write ``_f`` / ``_mark`` of every call (None: what ``set_export`` set in this thread)."""
+    export = export_enabled() if export is None else bool(export)
+    built = [_problem(c[0], c[1], c[2], c[3], c[5], c[6], c[7], c[8], c[9], export) for c in calls]
     _lib.solve_batch([b[1] for b in built])
-    return [_finish(keys, prob, c[4], c[5], c[10], _export) for (keys, prob), c in zip(built, calls)]
+    return [_finish(keys, prob, c[4], c[5], c[10], export) for (keys, prob), c in zip(built, calls)]

@@ -212,6 +212,22 @@ int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_c
  * into that state (1) or ends it (0) without a launch having to time out. */
 void gdp_debug_shared_device(int32_t seems_shared);
 
+/* Benchmark aid (no counterpart in the reference): what the gdp_solve_batch calls of the whole process did
+ * between gdp_batch_stats_begin() and gdp_batch_stats_end().  While it is on, every part of a batch is
+ * bracketed by two HIP events on its stream; device_ms is the sum of those intervals (first kernel of the
+ * part to its last one: relaxation launches and backtrack), so the host's share of a sweep's wall time is
+ * what is left of the wall clock. */
+typedef struct gdp_batch_stats {
+    double relaxations;   /* sum over the solved instances of L*V*S*S                      */
+    double executed;      /* of those, carried out (see gdp_timing.executed)               */
+    double device_ms;     /* sum over the parts of first kernel -> last kernel              */
+    int64_t instances;
+    int64_t parts;        /* plans (a batch above GALVATRON_DP_ARENA_MB is solved in parts) */
+    int64_t flow_parts, fused_parts, per_layer_parts; /* by launch scheme of the run        */
+} gdp_batch_stats;
+void gdp_batch_stats_begin(void);
+int gdp_batch_stats_end(gdp_batch_stats *out);
+
 /* Text of the calling thread's last error ("" if none). */
 const char *gdp_last_error(void);
 /* GDP_VERSION of the built library. */

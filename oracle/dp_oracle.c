@@ -16,7 +16,11 @@
  *   dp_oracle_epilogue  (csrc/dp_core.cpp:78-117) pinned: same tests, plus
  *       the memory/cost identities along the returned path.
  *   dp_oracle_coarse    (galvatron/core/search_engine/dynamic_programming.py:62-75)
- *       pinned: closed form (plain left-to-right sums) in tests.
+ *       pinned: on every coarse instance of the two coarse-mode scenarios whose
+ *       results were recorded from the reference's own DpOnModel
+ *       (tests/golden/dp_on_model_golden.json) it must give what the host
+ *       class gives, and the run as a whole the recorded tuples
+ *       (tests/test_oracle_pins.py::test_coarse_branch_against_the_reference_scenarios).
  *
  * Semantics restated (all from csrc/dp_core.cpp unless noted):
  *   - one f[V][S] buffer updated in place, v descending, s ascending (:57-59);

@@ -169,3 +169,29 @@ def test_static_entry_point_links_against_nothing_that_allocates(tmp_path):
                    "gdp_launch_init", "gdp_launch_relax", "gdp_launch_zero_pass", "gdp_launch_epilogue"}
     own = {n.split("(")[0] for n in names if n.startswith("gdp_")}
     assert own <= allowed_own, own - allowed_own
+
+
+def test_export_switch_is_per_thread():
+    """The reference's parallel search calls the plugin from many threads: a thread that asks for ``_f`` /
+    ``_mark`` to be written back must not change what the other threads allocate and copy."""
+    import threading
+
+    import galvatron_dp_core as shim
+    seen = {}
+
+    def worker():
+        seen["before"] = shim.export_enabled()
+        shim.set_export(True)
+        seen["after"] = shim.export_enabled()
+
+    assert shim.export_enabled() is False
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert seen == {"before": False, "after": True}
+    assert shim.export_enabled() is False
+    shim.set_export(True)
+    try:
+        assert shim.export_enabled() is True
+    finally:
+        shim.set_export(False)

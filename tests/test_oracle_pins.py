@@ -215,3 +215,39 @@ def test_coarse_branch_closed_form():
             assert list(res[k]) == [arg] * L and rem[k] == V - 1 - (int(mem[:, arg].sum()) + om[k])
         else:
             assert rem[k] == -1
+
+
+@pytest.mark.parametrize("name", ["flush_coarse", "flush_coarse_tight"])
+def test_coarse_branch_against_the_reference_scenarios(name, monkeypatch):
+    """What pins ``dp_oracle_coarse``: the two coarse-mode scenarios whose return tuples were written from
+    the reference's own ``DpOnModel`` (tests/golden/dp_on_model_golden.json).  Every coarse instance of
+    such a run is also handed to the C function, which must give what the host class gives -- and the
+    run as a whole must give the reference's recorded tuples.  (Coarse mode never reaches the plugin:
+    no device is needed.)"""
+    import json
+    import os
+
+    import dp_on_model_stubs as stubs
+    from galvatron_dp.dynamic_programming import DPAlg, DpOnModel
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "dp_on_model_golden.json")) as fh:
+        want = json.load(fh)[name]
+    seen = []
+    plain = DPAlg._fit_coarse
+
+    def checked(self):
+        total, res, rem = plain(self)
+        wt, wr, wm = O.coarse(self.v_data, self.intra_cost, np.asarray(self.inter_cost), self.max_mem,
+                              [s[1] for s in self.strategy_set], self.other_mem_cost, self.other_time_cost)
+        for k in self.other_mem_cost:
+            assert np.float64(total[k]).tobytes() == np.float64(wt[k]).tobytes(), (k, total[k], wt[k])
+            assert int(rem[k]) == int(wm[k]) and [int(x) for x in res[k]] == [int(x) for x in wr[k]]
+        seen.append(len(self.other_mem_cost))
+        return total, res, rem
+
+    monkeypatch.setattr(DPAlg, "_fit_coarse", checked)
+    cfg = stubs.scenario(name)
+    dpm = stubs.build(DpOnModel, cfg, other_timecost_model=stubs.StubOther, pipeline_costmodel=stubs.stub_pipeline_costmodel)
+    assert stubs.run(dpm, cfg) == want
+    assert len(seen) >= 3, "the scenario should have gone through the coarse branch for every stage"
