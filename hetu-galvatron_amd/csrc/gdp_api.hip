@@ -320,9 +320,24 @@ void fused_turn_take()
 // orders the threads of this process only).  Every further launch of that kind would risk the same
 // wait of a good part of a second, so for the next while the library chooses launches that never wait
 // (one per layer) where the choice is its own; a caller's explicit request still counts.
-constexpr int64_t DEFAULT_SPIN_LIMIT = 1 << 18;
-constexpr double SHARED_DEVICE_BACKOFF_S = 30.0;
+// How long a waiting wave keeps polling before its launch is given up, when the caller has set no limit of
+// its own: WAIT_BOUND_FACTOR times what the plan's relaxations take at a rate every healthy launch exceeds
+// (a wave of a healthy launch waits for less than the launch lasts), no less than WAIT_BOUND_MIN_S and no
+// more than WAIT_BOUND_MAX_S.  A solve of 0.1 ms gives up after 5 ms, one of 3 ms after a quarter of a second.
+constexpr double WAIT_BOUND_FACTOR = 50.0, WAIT_BOUND_RATE = 5e12 /* relaxations per second */;
+constexpr double WAIT_BOUND_MIN_S = 5e-3, WAIT_BOUND_MAX_S = 1.0;
+// Time between two looks of a waiting wave: a sleep of 3.5 us in a launch with completion counters; the round
+// trip of an agent-scope load, at least 1 us, in a flow launch (see wait_tiles and flow_poll in gdp_kernels.hip).
+constexpr double POLL_S_FUSED = 3.5e-6, POLL_S_FLOW = 1e-6;
 std::atomic<int64_t> g_last_give_up_ms{-1};   // steady clock, milliseconds; -1: never
+
+// For how long after a give-up launches that wait are avoided (GALVATRON_DP_SHARED_BACKOFF_MS; default 30 s).
+int64_t shared_backoff_ms()
+{
+    const char *e = getenv("GALVATRON_DP_SHARED_BACKOFF_MS");
+    if (e && *e) return std::max<long long>(0, atoll(e));
+    return 30000;
+}
 
 int64_t steady_ms()
 {
@@ -332,7 +347,7 @@ int64_t steady_ms()
 bool device_seems_shared()
 {
     const int64_t t = g_last_give_up_ms.load(std::memory_order_relaxed);
-    return t >= 0 && (double)(steady_ms() - t) < SHARED_DEVICE_BACKOFF_S * 1e3;
+    return t >= 0 && steady_ms() - t < shared_backoff_ms();
 }
 
 bool fused_turn_try_take()
@@ -540,8 +555,12 @@ struct gdp_plan {
     int flow_override = -1;       // GALVATRON_DP_FLOW=0|1: never / wherever the layout allows
     bool keep_marks = false;      // store the argmin table while relaxing (two cost buffers are then enough);
                                   // otherwise all L+1 cost buffers are kept and the backtrack recomputes it
-    int64_t spin_limit = DEFAULT_SPIN_LIMIT; // polls a waiting wave makes before the launch is abandoned: about a second
-                                  // (3.5 us apart), a thousand times the longest wait of a healthy launch
+    int64_t spin_limit = 0;       // polls a waiting wave makes before the launch is abandoned, if the caller has set
+                                  // them (GDP_OPT_SPIN_LIMIT, GALVATRON_DP_SPIN_LIMIT); 0: from wait_bound_s
+    double wait_bound_s = WAIT_BOUND_MAX_S;  // ... else for this long (set from the plan's size when it is laid out)
+    bool scheme_fused = false, scheme_flow = false;  // the launch scheme the plan was given (fused / flow are what it
+                                  // runs with now: both off after a give-up, until the plan is armed again)
+    int64_t gave_up_ms = -1;      // when a waiting launch of this plan was last given up (steady clock)
     size_t off_zero = 0, zero_words = 0, off_abort = 0;
     int num_cu = 0;
     size_t lds_per_cu = 0;
@@ -549,6 +568,7 @@ struct gdp_plan {
     bool rezero = false;     // buffer 0 is overwritten during a run and must be zeroed before each
     bool fused_gave_up = false;  // a fused launch was abandoned and the plan switched to per-layer launches
     bool no_fallback = false;    // GDP_OPT_NO_FALLBACK: report that instead of switching (tests)
+    bool debug_stall = false;    // GDP_OPT_DEBUG_STALL: the first layer of a waiting launch does not signal (tests)
     bool no_occupancy_cap = false;  // GALVATRON_DP_OCCUPANCY_CAP=0 (tuning aid)
     int occupancy_cap_override = 0; // GALVATRON_DP_OCCUPANCY_CAP=n: n workgroups per CU in fused launches
     int chunk_override = 0;         // GALVATRON_DP_CHUNK=n: n instances at a time in fused launches
@@ -1478,7 +1498,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             g.slots = (int)((widest + 7) / 8 * g.xcd_group);
         }
         sc->slots = g.slots;
-        sc->spin_limit = pl->spin_limit;
+        sc->spin_limit = 0;   // (set per launch: wait_polls)
         int32_t *act = reinterpret_cast<int32_t *>(stage.data() + g.off_active);
         for (int l = 0; l < g.max_L; ++l) act[l] = g.active[(size_t)l];
         sc->rows = nullptr;
@@ -1539,6 +1559,9 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
+    pl->scheme_fused = pl->fused;
+    pl->scheme_flow = pl->flow;
+    pl->wait_bound_s = std::min(WAIT_BOUND_MAX_S, std::max(WAIT_BOUND_MIN_S, WAIT_BOUND_FACTOR * pl->executed / WAIT_BOUND_RATE));
     if (pl->dry) {
         pl->inst.swap(inst);
         return GDP_OK;
@@ -1808,6 +1831,13 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
     GdpDevOut *d_out = reinterpret_cast<GdpDevOut *>(pl->dbase + pl->off_out);
     int32_t *d_res = reinterpret_cast<int32_t *>(pl->dbase + pl->off_res);
     pl->run_flow = false;
+    // A plan that gave a waiting launch up runs with one launch per layer -- until the time has passed for which
+    // the library avoids such launches after a give-up; then it is armed again with the scheme it was given.
+    if (pl->fused_gave_up && !pl->no_fallback && steady_ms() - pl->gave_up_ms >= shared_backoff_ms() && !device_seems_shared()) {
+        pl->fused_gave_up = false;
+        pl->fused = pl->scheme_fused;
+        pl->flow = pl->scheme_flow;
+    }
     if (pl->fused && !pl->holds_fused) {
         fused_turn_take();  // until run_finish has waited for the launch
         pl->holds_fused = true;
@@ -1840,6 +1870,9 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
         }
     }
     size_t li = 0;
+    auto wait_polls = [&](double poll_s) {
+        return pl->spin_limit > 0 ? pl->spin_limit : std::max<int64_t>(1, (int64_t)(pl->wait_bound_s / poll_s));
+    };
 
     if (pl->fused) {
         GDP_HIP(gdp_launch_zero(reinterpret_cast<int32_t *>(pl->dbase + pl->off_zero), (int64_t)pl->zero_words,
@@ -1848,8 +1881,11 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             for (const auto &seg : g.segments) {
                 const int grid_x = 8 * (g.rows.empty() ? g.active[(size_t)seg.first] : g.chunk) * g.slots;
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
+                GdpSched sched = g.sched;
+                sched.spin_limit = wait_polls(POLL_S_FUSED);
+                sched.debug_stall = pl->debug_stall ? 1 : 0;
                 GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
-                                               g.sched, grid_x,
+                                               sched, grid_x,
                                                seg.first, seg.layers, seg.lds_bytes, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
                 ++li;
@@ -1863,7 +1899,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li], pl->stream));
             if (g.flow_blocks > 0)
                 GDP_HIP(gdp_launch_relax_flow(g.flow_nsrc, g.latency, g.sched.lay, g.max_L, g.count, g.flow_blocks, g.SP, 0, g.max_L,
-                                              g.sched.abort_flag, pl->spin_limit, pl->stream));
+                                              g.sched.abort_flag, wait_polls(POLL_S_FLOW), pl->debug_stall, pl->stream));
             if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
             ++li;
         }
@@ -1925,7 +1961,9 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
         pl->fused = false;
         pl->flow = false;
         pl->fused_gave_up = true;
-        if (pl->spin_limit >= DEFAULT_SPIN_LIMIT) g_last_give_up_ms.store(steady_ms(), std::memory_order_relaxed);
+        pl->gave_up_ms = steady_ms();
+        // nobody had shortened the waits: something else holds places on the device
+        if (pl->spin_limit == 0) g_last_give_up_ms.store(pl->gave_up_ms, std::memory_order_relaxed);
         if (pl->no_fallback)
             return fail(GDP_E_HIP, "fused launch: a bounded wait ran out before its tiles were finished");
         return run(pl, mode, t);
@@ -2086,14 +2124,16 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
         case GDP_OPT_FUSED:
             if (value != 0 && !plan->can_fuse)
                 return fail(GDP_E_BADARG, "plan was laid out for per-layer launches only (two cost buffers, or a memory cost of 0)");
-            plan->fused = value != 0;
-            plan->flow = false;
+            plan->fused = plan->scheme_fused = value != 0;
+            plan->flow = plan->scheme_flow = false;
+            plan->fused_gave_up = false;
             return GDP_OK;
         case GDP_OPT_FLOW:
             if (value != 0 && !plan->flow_ready)
                 return fail(GDP_E_BADARG, "plan was not laid out for a flow launch (see GALVATRON_DP_FLOW)");
-            plan->flow = value != 0;
-            if (plan->flow) plan->fused = false;
+            plan->flow = plan->scheme_flow = value != 0;
+            if (plan->flow) plan->fused = plan->scheme_fused = false;
+            plan->fused_gave_up = false;
             return GDP_OK;
         case GDP_OPT_POISON:
             plan->poison = value != 0;
@@ -2101,11 +2141,12 @@ int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value)
         case GDP_OPT_NO_FALLBACK:
             plan->no_fallback = value != 0;
             return GDP_OK;
+        case GDP_OPT_DEBUG_STALL:
+            plan->debug_stall = value != 0;
+            return GDP_OK;
         case GDP_OPT_SPIN_LIMIT: {
             if (value < 1) return fail(GDP_E_BADARG, "spin limit must be >= 1");
             plan->spin_limit = value;
-            GDP_HIP(hipSetDevice(plan->device));
-            for (Group &g : plan->groups) g.sched.spin_limit = value;
             return GDP_OK;
         }
         default:

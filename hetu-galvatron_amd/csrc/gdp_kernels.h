@@ -100,6 +100,8 @@ struct GdpSched {
     int32_t group;            // consecutive block tasks that go to one XCD (whole tiles)
     int32_t slots;            // workgroups per XCD, instance and layer: ceil(ceil(block tasks / group) / 8) * group
     int64_t spin_limit;       // polls before a waiting wave gives up
+    int32_t debug_stall;      // test aid: tasks of layer 0 do not signal their completion, so that every wait for
+                              // them runs into its bound (the launch drains, the host repeats the solve)
 };
 
 struct GdpDevKey {
@@ -163,8 +165,11 @@ static const int GDP_FLOW_NSRC[] = {8, 12, 16, 20, 24, 28, 32};
 // layers' SU being nsrc * latency).  grid_blocks: workgroups of the widest band.
 // The cells the launch writes must hold NaN beforehand and the abort flag zero: gdp_launch_flow_reset
 // (bands of all layers of n_inst instances).
+// debug_stall: test aid -- the tasks of layer 0 leave their stores out, so that every wait for them runs into
+// its bound.
 hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
-                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, hipStream_t stream);
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, bool debug_stall,
+                                 hipStream_t stream);
 hipError_t gdp_launch_flow_reset(const GdpDevInst *insts, int n_inst, int64_t max_ld, int max_S, const GdpDevLayer *lay,
                                  int max_L, int tile_rows, int32_t *abort_flag, hipStream_t stream);
 // Sets up H.  what = GDP_INIT_PADS: +inf pads and +inf row of every buffer (once per plan);

@@ -373,7 +373,7 @@ __device__ __forceinline__ FlowHead load_flow_head(const GdpDevLayer *Y)
 //     agent scope: S=44 V=32768 L=32 0.44 instead of 0.38 ms, S=40 V=29493 L=28 0.22 instead of 0.19.)
 template <int TS, int NSRC, int K>
 __device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile, unsigned vtb, unsigned lane,
-                                                FlowWait &w)
+                                                FlowWait &w, bool stall)
 {
     static_assert(K == 1 || GDP_WAVES_PER_BLOCK % K == 0, "parts of one task share a workgroup");
     static_assert(TS <= 16, "a row of 16 lanes holds the transition costs of a step");
@@ -499,7 +499,7 @@ __device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile
 #pragma unroll
     for (int j = 0; j < TS; ++j) {
         if (j < nvalid) {
-            if (mine[j])
+            if (mine[j] && !stall)
                 __hip_atomic_store(drow + lane, best[0][j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             drow += ld;
         }
@@ -930,7 +930,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
                                                               // are filled or skipped there and count as done
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every write-through store acknowledged
-    if (lane == 0)
+    if (lane == 0 && !(Q.debug_stall && layer == 0))
         __hip_atomic_fetch_add(cnt_all + ((int64_t)ii * max_L + layer) * max_ntile + tile, 1, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -955,7 +955,8 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
 // l-1's output lies in that layer's band, below it (filled once per plan) or in the pads.
 template <int NSRC, int K>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 8 / GDP_WAVES_PER_BLOCK) void gdp_relax_flow_kernel(
-    const GdpDevLayer *__restrict__ lay, int max_L, int layer0, unsigned ntb, int32_t *abort_flag, int64_t spin_limit)
+    const GdpDevLayer *__restrict__ lay, int max_L, int layer0, unsigned ntb, int32_t *abort_flag, int64_t spin_limit,
+    int debug_stall)
 {
     const GdpDevLayer *Y = lay + ((int64_t)blockIdx.z * max_L + layer0 + (int)blockIdx.y);
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -966,7 +967,8 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 8 / GDP_WAVES_PER_BLOCK) 
     if (task >= live_tasks) return;
     const unsigned t = task / ntb;
     FlowWait fw = {abort_flag, spin_limit, 0, false};
-    relax_task_flow<GDP_LAT_TS, NSRC, K>(H, (unsigned)H.lo + t, task - t * ntb, lane, fw);
+    relax_task_flow<GDP_LAT_TS, NSRC, K>(H, (unsigned)H.lo + t, task - t * ntb, lane, fw,
+                                         debug_stall != 0 && layer0 + (int)blockIdx.y == 0);
 }
 
 // NaN into every cell that a flow launch writes (the bands of all layers), and zero into its abort flag.
@@ -1520,7 +1522,8 @@ hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched
 }
 
 hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, int max_L, int n_inst, int grid_blocks, int SP,
-                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, hipStream_t stream)
+                                 int layer0, int layers, int32_t *abort_flag, int64_t spin_limit, bool debug_stall,
+                                 hipStream_t stream)
 {
     if (n_inst < 1 || n_inst > 65535 || layers < 1 || layers > 65535 || grid_blocks < 1) return hipErrorInvalidValue;
     const unsigned ntb = (unsigned)(SP / GDP_LAT_TS) * (unsigned)latency;  // with the parts of a split task
@@ -1528,7 +1531,7 @@ hipError_t gdp_launch_relax_flow(int nsrc, int latency, const GdpDevLayer *lay, 
 #define X(NSRC, K)                                                                                                   \
     if (nsrc == NSRC && latency == K) {                                                                              \
         hipLaunchKernelGGL((gdp_relax_flow_kernel<NSRC, K>), grid, block, 0, stream, lay, max_L, layer0, ntb, \
-                           abort_flag, spin_limit);                                                                  \
+                           abort_flag, spin_limit, debug_stall ? 1 : 0);                                             \
         return hipGetLastError();                                                                                    \
     }
     GDP_FOR_EACH_FLOW(X)

@@ -34,6 +34,7 @@ GDP_OPT_SPIN_LIMIT = 2
 GDP_OPT_POISON = 3
 GDP_OPT_NO_FALLBACK = 4
 GDP_OPT_FLOW = 5
+GDP_OPT_DEBUG_STALL = 6
 
 GDP_STATIC_SCRATCH_BYTES = 64 << 20
 

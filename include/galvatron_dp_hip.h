@@ -177,7 +177,11 @@ void gdp_plan_destroy(gdp_plan *plan);
  *                      buffers that did not fit in device memory) cannot be switched to 1.
  *   GDP_OPT_SPIN_LIMIT polls a waiting wavefront makes before it gives up; when that happens the
  *                      launch drains normally, the plan switches itself to one launch per layer
- *                      and the run is repeated that way (GDP_E_HIP with GDP_OPT_NO_FALLBACK). */
+ *                      and the run is repeated that way (GDP_E_HIP with GDP_OPT_NO_FALLBACK).  Default: a
+ *                      time, not a count -- 50 times what the plan's relaxations take at 5e12 per second,
+ *                      between 5 ms and 1 s -- turned into polls per launch scheme.  A plan that gave up
+ *                      is armed again with its launch scheme once GALVATRON_DP_SHARED_BACKOFF_MS (default
+ *                      30000) have passed. */
 #define GDP_OPT_FUSED 1
 #define GDP_OPT_SPIN_LIMIT 2
 #define GDP_OPT_POISON 3 /* test aid: NaN-fill every not-yet-written cost buffer before each run */
@@ -187,6 +191,10 @@ void gdp_plan_destroy(gdp_plan *plan);
                           for rows that are not whole yet.  Chosen by the library for plans too small for
                           GDP_OPT_FUSED to pay (unless a launch scheme was asked for); only a plan laid out for it
                           can be switched to 1.  0: one launch per layer.  Waits are bounded like GDP_OPT_FUSED's. */
+#define GDP_OPT_DEBUG_STALL 6 /* test aid: in launches whose workgroups wait (GDP_OPT_FUSED, GDP_OPT_FLOW) the tasks of
+                                 the first layer leave out the signal the next layer waits for, so that every such wait
+                                 runs into its bound: the launch drains, every kernel ends normally, and the solve is
+                                 repeated with one launch per layer */
 int gdp_plan_set_option(gdp_plan *plan, int32_t option, int64_t value);
 
 /* Frees the device allocations that finished plans left behind for reuse (no counterpart in the
@@ -207,7 +215,7 @@ int gdp_debug_check_layout(int32_t n, const gdp_problem *const *p, int32_t num_c
 
 /* Test aid (no counterpart in the reference).  After a launch whose workgroups wait (GDP_OPT_FUSED,
  * GDP_OPT_FLOW) has been given up with the default spin limit, the library takes the device to be shared
- * with another process and, for the next 30 seconds, chooses one launch per layer wherever the choice is
+ * with another process and, for the next 30 seconds (GALVATRON_DP_SHARED_BACKOFF_MS), chooses one launch per layer wherever the choice is
  * its own (explicit requests -- flags, options, environment -- still count).  This call puts the library
  * into that state (1) or ends it (0) without a launch having to time out. */
 void gdp_debug_shared_device(int32_t seems_shared);

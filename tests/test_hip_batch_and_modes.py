@@ -346,6 +346,39 @@ def test_abandoned_fused_launch_falls_back_or_reports(golden):
     _check_against_golden(prob3, rec, "after")
 
 
+def test_a_wait_that_cannot_end_costs_milliseconds_and_the_plan_is_armed_again(golden, monkeypatch):
+    """The first layer of the fused launch leaves its completion counters alone (forced from the host; every
+    kernel still ends normally), so the waits of the second layer run into their bound.  That bound follows
+    from the plan's size -- 5 ms for a plan this small, where a fixed number of polls used to take a second --
+    after which the solve is repeated with one launch per layer and gives the right answer.  Once the time has
+    passed for which the library avoids waiting launches, the plan runs with its own launch scheme again."""
+    import time
+    rec = golden["cfg2_small"]
+    inst = H.build_case(rec)
+    monkeypatch.setenv("GALVATRON_DP_SHARED_BACKOFF_MS", "150")
+    prob = _problem(inst, launch="fused")
+    try:
+        with _lib.Plan([prob]) as plan:
+            assert plan.run(1).fused == 1
+            plan.set_option(_lib.GDP_OPT_DEBUG_STALL, 1)
+            t0 = time.perf_counter()
+            t = plan.run(1)
+            dt = time.perf_counter() - t0
+            plan.fetch()
+            _check_against_golden(prob, rec, "after the bounded wait ran out")
+            assert t.fused == 0 and t.relax_launches == inst.L
+            assert dt < 0.25, f"give-up and repeated solve took {dt * 1e3:.0f} ms"
+            plan.set_option(_lib.GDP_OPT_DEBUG_STALL, 0)
+            assert plan.run(1).fused == 0                  # still inside the back-off: one launch per layer
+            time.sleep(0.3)
+            t = plan.run(1)
+            plan.fetch()
+            assert t.fused == 1, "the plan was not armed again after the back-off"
+            _check_against_golden(prob, rec, "armed again")
+    finally:
+        _lib.debug_shared_device(False)
+
+
 def test_shim_batch_entry_point(golden):
     import galvatron_dp_core as shim
     names = ["rand_1", "ties_3", "infeasible_5"]

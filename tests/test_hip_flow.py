@@ -159,6 +159,39 @@ def test_abandoned_flow_launch_falls_back_or_reports(golden):
     _check_against_golden(prob3, rec, "after")
 
 
+def test_a_flow_wait_that_cannot_end_costs_milliseconds(golden, monkeypatch):
+    """The tasks of the first layer leave their stores out (forced from the host; every kernel still ends
+    normally), so the second layer waits for cells that stay unwritten until the bound of the wait -- 5 ms for
+    a plan of this size -- runs out; the solve is then repeated with one launch per layer, and after the
+    back-off the plan flows again."""
+    import time
+    if any(k in os.environ for k in _PRESETS):
+        pytest.skip("the environment presets the layout")
+    rec = golden["cfg0"]
+    inst = H.build_case(rec)
+    monkeypatch.setenv("GALVATRON_DP_SHARED_BACKOFF_MS", "150")
+    prob = _problem(inst)
+    try:
+        with _lib.Plan([prob]) as plan:
+            assert plan.run(1).flow == 1
+            plan.set_option(_lib.GDP_OPT_DEBUG_STALL, 1)
+            t0 = time.perf_counter()
+            t = plan.run(1)
+            dt = time.perf_counter() - t0
+            plan.fetch()
+            _check_against_golden(prob, rec, "after the bounded wait ran out")
+            assert t.flow == 0 and t.relax_launches == inst.L
+            assert dt < 0.25, f"give-up and repeated solve took {dt * 1e3:.0f} ms"
+            plan.set_option(_lib.GDP_OPT_DEBUG_STALL, 0)
+            time.sleep(0.3)
+            t = plan.run(1)
+            plan.fetch()
+            assert t.flow == 1, "the plan was not armed again after the back-off"
+            _check_against_golden(prob, rec, "armed again")
+    finally:
+        _lib.debug_shared_device(False)
+
+
 def test_flow_plans_from_several_threads(golden):
     """Threads that call the plugin side by side (as the reference's parallel search does): one flow
     launch runs at a time, a plan that finds the turn taken solves with one launch per layer beside
