@@ -849,18 +849,67 @@ int upload_f0(gdp_plan *pl)
     return GDP_OK;
 }
 
-// f0_live: null, or per problem whether its f0 holds anything but zeros (validate_all).
-int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks, const char *f0_live)
+// Lays a plan out and brings it onto the device, one step after the other (create() below runs them in order).
+// What more than one step needs lives here; everything that outlasts the creation is written into the plan.
+struct PlanBuilder {
+    int32_t n;
+    const gdp_problem *const *p;
+    gdp_plan *pl;
+    bool force_marks;      // start over with the argmin table (the costs-only layout did not fit the device)
+    const char *f0_live;   // null, or per problem whether its f0 holds anything but zeros (validate_all)
+
+    bool fused_preset = false;   // the launch scheme was asked for (environment, flags): it is not the library's choice
+    bool marks_preset = false;
+    std::vector<HostInst> inst;  // sorted by S, then by L descending; moved into the plan at the end
+    int64_t wave_slots = 0;      // wave slots of the device at 4 resident waves per SIMD
+    double band_frac = 1.0;      // share of the relaxations that lie inside the bands
+    size_t off = 0;              // next free byte of the device allocation while it is laid out
+    int nk = 0;                  // keys / strategy-list entries of all instances
+    size_t nres = 0;
+    size_t small_bytes = 0;      // tables and per-instance inputs: what is built on the host and uploaded
+    size_t fixed_bytes = 0;      // ... plus counters and results: everything in front of the cost buffers
+    int max_S = 0;
+    struct { char *p; char *data() const { return p; } } stage = {nullptr};   // host copy of the first small_bytes
+    std::vector<std::vector<int32_t>> h_band;   // per instance {tiles a reader reaches down, first, last tile to compute} per layer
+    bool turn_free = false;      // a flow plan whose first run will most likely flow (nobody holds the turn)
+    bool prepared_early = false; // ... and whose cost buffers are already being prepared by a kernel fed with arguments
+    GdpDevInst *di = nullptr;    // instance and key records inside `stage`
+    GdpDevKey *dk = nullptr;
+
+    size_t take(size_t bytes)
+    {
+        const size_t o = off;
+        off = align_up(off + bytes, 256);
+        return o;
+    }
+    int read_presets();
+    int describe_device();
+    void describe_instances();
+    int form_groups();
+    struct FlowPick { int K, nsrc; double resident; };
+    FlowPick flow_pick(const Group &g) const;
+    void choose_launch_scheme();
+    int lay_out_tables();
+    int allocate();
+    int take_stage();
+    void compute_bands();
+    int32_t fill_from_of(int i, int l) const;
+    int prepare_early();
+    void build_instance_tables();
+    void build_group_tables();
+    int upload();
+};
+
+// Options of the plan: presets from the environment, then what the problems' flags ask for.
+int PlanBuilder::read_presets()
 {
     pl->n = n;
     if (!pl->dry) GDP_HIP(hipGetDevice(&pl->device));
     // defaults of the plan options can be preset from the environment
-    bool fused_preset = false;
     if (const char *e = getenv("GALVATRON_DP_FUSED")) {
         pl->fused = atoi(e) != 0;
         fused_preset = true;
     }
-    bool marks_preset = false;
     if (const char *e = getenv("GALVATRON_DP_KEEP_MARKS")) {
         pl->keep_marks = atoi(e) != 0;
         marks_preset = true;
@@ -899,7 +948,12 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->fused = false;    // (mem == 0: a cell then depends on cells of its own layer, which the counters of a
         fused_preset = true;  //  fused launch do not order)
     }
-    // ---- shapes -------------------------------------------------------------------------------
+    return GDP_OK;
+}
+
+// Compute units and LDS per unit of the device the plan is for.
+int PlanBuilder::describe_device()
+{
     if (pl->dry) {
         pl->num_cu = pl->dry_num_cu;
         pl->lds_per_cu = pl->dry_lds_per_cu;
@@ -917,7 +971,13 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->num_cu = known[(size_t)pl->device].first;
         pl->lds_per_cu = known[(size_t)pl->device].second;
     }
-    std::vector<HostInst> inst((size_t)n);
+    return GDP_OK;
+}
+
+// Shapes of the instances, their equal transition matrices, their initial costs; sorted into groups of one S.
+void PlanBuilder::describe_instances()
+{
+    inst.assign((size_t)n, HostInst());
     for (int i = 0; i < n; ++i) {
         const gdp_problem *q = p[i];
         HostInst &h = inst[(size_t)i];
@@ -945,7 +1005,12 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         if (a.S != b.S) return a.S < b.S;
         return a.L > b.L;
     });
-    const int64_t wave_slots = (int64_t)pl->num_cu * 4 * 4;  // 4 SIMDs x 4 resident waves
+}
+
+// One group per S: register tile, chunking of fused launches, row lengths, per-layer activity.
+int PlanBuilder::form_groups()
+{
+    wave_slots = (int64_t)pl->num_cu * 4 * 4;  // 4 SIMDs x 4 resident waves
     for (int i = 0; i < n;) {
         Group g;
         g.first = i; g.S = inst[(size_t)i].S;
@@ -1038,7 +1103,13 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->groups.push_back(g);
         i = j;
     }
-    double band_frac = 1.0;   // share of the relaxations that lie inside the bands
+    return GDP_OK;
+}
+
+// Which of the three launch schemes the plan runs with, where the caller has not said (see the comments
+// inside), and with it the variant of the per-layer kernel and how a task's sources are split over waves.
+void PlanBuilder::choose_launch_scheme()
+{
     if (!fused_preset || pl->flow_override != 0) {
         // One launch for all layers pays off once a layer holds about two block tasks that carry
         // arithmetic per CU (measured: 950 per layer, 0.48 ms against 0.58 ms; 128 per layer, 0.23 ms
@@ -1080,29 +1151,6 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     // (forced onto the narrow tile and the flow launch: S=44 V=65536 L=32 0.63 against 0.64 ms, S=44
     // V=131072 1.22 against 0.83, S=64 V=65536 L=16 0.62 against 0.45).  GALVATRON_DP_FLOW=1 asks for it
     // wherever the layout allows (costs only, no memory cost of 0, the tile of the latency variant).
-    struct FlowPick { int K, nsrc; double resident; };
-    auto flow_pick = [&](const Group &g) {
-        auto waves_per_simd = [](int nsrc) { return nsrc <= 12 ? 8 : nsrc <= 16 ? 7 : nsrc <= 20 ? 6 : nsrc <= 28 ? 5 : 4; };  // by their registers (38 + 2 per source)
-        auto nsrc_for = [&](int K) {
-            for (int c : GDP_FLOW_NSRC)
-                if (c * K >= g.S) return c;
-            return 0;
-        };
-        double band_tiles = 0;   // of an average layer, over the group
-        for (int k = g.first; k < g.first + g.count; ++k) band_tiles += (double)inst[(size_t)k].ntile * band_frac;
-        const int ntb8 = (g.S + GDP_LAT_TS - 1) / GDP_LAT_TS;
-        FlowPick best = {0, 0, -1.0};
-        for (int K : {4, 2, 1}) {
-            const int c = nsrc_for(K);
-            if (!c) continue;
-            const double res = (double)pl->num_cu * 4 * waves_per_simd(c) / std::max(1.0, band_tiles * ntb8 * K);
-            if (pl->latency_override >= 1 && K == (pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1))
-                return FlowPick{K, c, res};
-            if (res >= 2.0 && best.resident < 2.0) best = {K, c, res};
-            if (best.resident < 2.0 && res > best.resident) best = {K, c, res};
-        }
-        return best;
-    };
     bool want_flow = pl->flow_override >= 0 ? pl->flow_override == 1 && !(fused_preset && pl->fused)
                                             : !fused_preset && !device_seems_shared();
     want_flow = want_flow && !pl->keep_marks && !pl->has_zero && pl->max_L <= 65534;
@@ -1141,15 +1189,43 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             for (int k = g.first; k < g.first + g.count; ++k) inst[(size_t)k].SU = su;
         }
     }
-    // ---- device layout: [tables | per-instance inputs] (uploaded in one copy) then [H, M] ------
-    size_t off = 0;
-    auto take = [&](size_t bytes) {
-        size_t o = off;
-        off = align_up(off + bytes, 256);
-        return o;
-    };
-    int nk = 0;
-    size_t nres = 0;
+}
+
+// Flow launch: waves per task (4, 2, 1) and sources per wave for a group -- the most waves that keep two
+// layers' tasks resident, else what keeps the most.
+PlanBuilder::FlowPick PlanBuilder::flow_pick(const Group &g) const
+{
+    {
+        auto waves_per_simd = [](int nsrc) { return nsrc <= 12 ? 8 : nsrc <= 16 ? 7 : nsrc <= 20 ? 6 : nsrc <= 28 ? 5 : 4; };  // by their registers (38 + 2 per source)
+        auto nsrc_for = [&](int K) {
+            for (int c : GDP_FLOW_NSRC)
+                if (c * K >= g.S) return c;
+            return 0;
+        };
+        double band_tiles = 0;   // of an average layer, over the group
+        for (int k = g.first; k < g.first + g.count; ++k) band_tiles += (double)inst[(size_t)k].ntile * band_frac;
+        const int ntb8 = (g.S + GDP_LAT_TS - 1) / GDP_LAT_TS;
+        FlowPick best = {0, 0, -1.0};
+        for (int K : {4, 2, 1}) {
+            const int c = nsrc_for(K);
+            if (!c) continue;
+            const double res = (double)pl->num_cu * 4 * waves_per_simd(c) / std::max(1.0, band_tiles * ntb8 * K);
+            if (pl->latency_override >= 1 && K == (pl->latency_override >= 4 ? 4 : pl->latency_override >= 2 ? 2 : 1))
+                return FlowPick{K, c, res};
+            if (res >= 2.0 && best.resident < 2.0) best = {K, c, res};
+            if (best.resident < 2.0 && res > best.resident) best = {K, c, res};
+        }
+        return best;
+    }
+}
+
+// Device layout, first part: [tables | per-instance inputs] (uploaded in one copy), then the words every run
+// resets and the results (copied back in one piece).
+int PlanBuilder::lay_out_tables()
+{
+    off = 0;
+    nk = 0;
+    nres = 0;
     {
         // the key table and the array of strategy lists are indexed with 32-bit offsets on the device
         size_t keys = 0, lists = 0;
@@ -1215,7 +1291,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         h.off_mem = take(sizeof(int32_t) * (size_t)h.L * h.S);
         h.off_zcols = h.has_zero ? take(sizeof(int32_t) * (size_t)h.L * (size_t)(h.S + 1)) : 0;
     }
-    const size_t small_bytes = off;
+    small_bytes = off;
     pl->small_bytes = small_bytes;
     // words that every fused run resets to zero: completion counters, abort flag
     pl->off_zero = off;
@@ -1228,11 +1304,17 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     pl->off_out = take(sizeof(GdpDevOut) * (size_t)std::max(nk, 1));
     pl->off_res = take(sizeof(int32_t) * std::max<size_t>(nres, 1));
     pl->back_bytes = off - pl->off_abort;
-    const size_t fixed_bytes = off;
+    fixed_bytes = off;
+    return GDP_OK;
+}
+
+// Device layout, second part: the cost buffers (and the argmin table), and the allocation itself.
+int PlanBuilder::allocate()
+{
     // One cost buffer per layer lets all layers share a launch and lets the backtrack recompute the
     // argmin of the cells it visits, so that the relaxation does not have to track it.  If that does
     // not fit in device memory: two cost buffers, the argmin table, one launch per layer.
-    int max_S = 0;
+    max_S = 0;
     for (const auto &h : inst) max_S = std::max(max_S, h.S);
     if (pl->keep_marks && max_S > GDP_MAX_S_MARKS)  // preset from the environment
         return fail(GDP_E_BADARG, "S exceeds GDP_MAX_S_MARKS and the argmin table is to be kept");
@@ -1266,7 +1348,12 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         snprintf(buf, sizeof buf, "hipMalloc of %zu bytes", pl->dbytes);
         return fail_hip(e, buf);
     }
-    // ---- build the small region on the host ------------------------------------------------------
+    return GDP_OK;
+}
+
+// Stream, events and page-locked buffers of the plan, and the host memory the tables are built in.
+int PlanBuilder::take_stage()
+{
     if (!pl->dry) {
         const hipError_t e = lane_take(pl->device, pl->back_bytes, small_bytes, &pl->lane);
         if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
@@ -1278,7 +1365,7 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->ev_begin = pl->lane.ev_begin;
         pl->ev_end = pl->lane.ev_end;
     }
-    struct { char *p; char *data() const { return p; } } stage = {pl->lane.up};
+    stage.p = pl->lane.up;
     if (small_bytes > UPLOAD_PINNED_MAX || pl->dry) {
         try {
             pl->stage.assign(small_bytes, 0);
@@ -1291,36 +1378,48 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         // the buffer any more
         memset(stage.p, 0, small_bytes);
     }
-    // {tiles a reader reaches down, first tile to compute, last tile to compute} per layer
-    std::vector<std::vector<int32_t>> h_band((size_t)n);
+    return GDP_OK;
+}
+
+// The band of tiles every layer of every instance has to compute.
+void PlanBuilder::compute_bands()
+{
+    h_band.assign((size_t)n, std::vector<int32_t>());
     for (int i = 0; i < n; ++i) {
         const HostInst &h = inst[(size_t)i];
         h_band[(size_t)i].assign((size_t)h.L * 3, 0);
         fill_bands(p[h.orig], h, 64 * GDP_VARIANTS[h.variant].r, pl->skip, h_band[(size_t)i].data(), &pl->executed,
                    pl->flow_ready);
     }
-    // Rows of a layer's output below its band are +inf and are filled once per plan -- those that something
-    // reads: the band of the next layer reaches down by at most this layer's largest memory cost (the
-    // backtrack reads what the relaxation read), the epilogue and the pass for memory costs of 0 read anywhere.
-    auto fill_from_of = [&](int i, int l) -> int32_t {
-        const HostInst &h = inst[(size_t)i];
-        if (l + 1 >= h.L || h.has_zero) return 0;
-        const int64_t lo_next = h_band[(size_t)i][3 * (size_t)(l + 1) + 1];
-        const int64_t reach = (int64_t)h_band[(size_t)i][3 * (size_t)l];   // tiles
-        return (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
-    };
-    // A small plan laid out for the flow launch, the turn free right now (its first run will most likely
-    // flow): the kernel that prepares its cost buffers -- pads, zeros, the filled rows, NaN into the bands --
-    // gets what it needs with its arguments and starts here, before the tables below have even been built;
-    // it runs beside the host's work on them and beside their upload (which then goes over the second stream
-    // in one piece).  (A Galvatron-like call: upload 15 us, then this kernel 42 us, then the first launch;
-    // now the kernel is under way 30 us earlier.)
-    bool turn_free = false;
+}
+
+// Rows of a layer's output below its band are +inf and are filled once per plan -- those that something
+// reads: the band of the next layer reaches down by at most this layer's largest memory cost (the
+// backtrack reads what the relaxation read), the epilogue and the pass for memory costs of 0 read anywhere.
+// The first such row of layer l of instance i.
+int32_t PlanBuilder::fill_from_of(int i, int l) const
+{
+    const HostInst &h = inst[(size_t)i];
+    if (l + 1 >= h.L || h.has_zero) return 0;
+    const int64_t lo_next = h_band[(size_t)i][3 * (size_t)(l + 1) + 1];
+    const int64_t reach = (int64_t)h_band[(size_t)i][3 * (size_t)l];   // tiles
+    return (int32_t)std::max<int64_t>(0, (lo_next - reach) * (64 * GDP_VARIANTS[h.variant].r));
+}
+
+// A small plan laid out for the flow launch, the turn free right now (its first run will most likely
+// flow): the kernel that prepares its cost buffers -- pads, zeros, the filled rows, NaN into the bands --
+// gets what it needs with its arguments and starts here, before the tables have even been built; it runs
+// beside the host's work on them and beside their upload (which then goes over the second stream in one
+// piece).  (A Galvatron-like call: upload 15 us, then this kernel 42 us, then the first launch; now the
+// kernel is under way 30 us earlier.)
+int PlanBuilder::prepare_early()
+{
+    turn_free = false;
     if (!pl->dry && pl->flow_ready) {
         std::lock_guard<std::mutex> lk(g_fused_mu);
         turn_free = !g_fused_busy;
     }
-    bool prepared_early = false;
+    prepared_early = false;
     if (turn_free && n <= GDP_PREP_MAX_INST) {
         int layers = 0;
         for (const auto &h : inst) layers += h.L;
@@ -1352,8 +1451,15 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
             prepared_early = true;
         }
     }
-    GdpDevInst *di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
-    GdpDevKey *dk = reinterpret_cast<GdpDevKey *>(stage.data() + pl->off_keys);
+    return GDP_OK;
+}
+
+// The host copy of the per-instance device tables: instance and key records, transition matrices, intra
+// costs, row offsets.
+void PlanBuilder::build_instance_tables()
+{
+    di = reinterpret_cast<GdpDevInst *>(stage.data() + pl->off_insts);
+    dk = reinterpret_cast<GdpDevKey *>(stage.data() + pl->off_keys);
     for (int i = 0; i < n; ++i) {
         const HostInst &h = inst[(size_t)i];
         const gdp_problem *q = p[h.orig];
@@ -1419,6 +1525,12 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
         pl->relaxations += (double)h.L * h.V * (double)h.S * h.S;
         pl->relax_bytes += (double)h.L * h.V * (double)h.S * (8 + 8 + (pl->keep_marks ? 1 : 0));
     }
+}
+
+// The host copy of the per-group tables: one record per (instance, layer), and what a fused launch needs --
+// slots per XCD, the runs of layers that share a launch, the occupancy cap of each.
+void PlanBuilder::build_group_tables()
+{
     // grid.y of a launch; GALVATRON_DP_MAX_GRID_ROWS lowers it (test aid: splits launches of small cases)
     int max_grid_rows = 65535;
     if (const char *e = getenv("GALVATRON_DP_MAX_GRID_ROWS")) max_grid_rows = std::min(65535, std::max(1, atoi(e)));
@@ -1559,13 +1671,11 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
         }
     }
-    pl->scheme_fused = pl->fused;
-    pl->scheme_flow = pl->flow;
-    pl->wait_bound_s = std::min(WAIT_BOUND_MAX_S, std::max(WAIT_BOUND_MIN_S, WAIT_BOUND_FACTOR * pl->executed / WAIT_BOUND_RATE));
-    if (pl->dry) {
-        pl->inst.swap(inst);
-        return GDP_OK;
-    }
+}
+
+// The tables onto the device, and the parts of the cost buffers that no run ever overwrites.
+int PlanBuilder::upload()
+{
     // A flow plan (small): the tables go first, the kernel that prepares the cost buffers needs nothing else;
     // the per-instance inputs follow on a second stream, beside that kernel.
     size_t tables_bytes = small_bytes;
@@ -1608,9 +1718,38 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
     }
     // no wait here: the stream orders the upload and these fills before the first run, the host copy
     // stays alive as long as the plan, and an error of theirs is reported by the run
-    pl->inst.swap(inst);
-    return upload_f0(pl);
+    return GDP_OK;
 }
+
+// f0_live: null, or per problem whether its f0 holds anything but zeros (validate_all).
+int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_marks, const char *f0_live)
+{
+    PlanBuilder b{n, p, pl, force_marks, f0_live};
+    int rc = b.read_presets();
+    if (rc == GDP_OK) rc = b.describe_device();
+    if (rc != GDP_OK) return rc;
+    b.describe_instances();
+    rc = b.form_groups();
+    if (rc != GDP_OK) return rc;
+    b.choose_launch_scheme();
+    rc = b.lay_out_tables();
+    if (rc == GDP_OK) rc = b.allocate();     // (may ask to start over with the argmin table: GDP_RETRY_WITH_MARKS)
+    if (rc == GDP_OK) rc = b.take_stage();
+    if (rc != GDP_OK) return rc;
+    b.compute_bands();
+    rc = b.prepare_early();
+    if (rc != GDP_OK) return rc;
+    b.build_instance_tables();
+    b.build_group_tables();
+    pl->scheme_fused = pl->fused;
+    pl->scheme_flow = pl->flow;
+    pl->wait_bound_s = std::min(WAIT_BOUND_MAX_S, std::max(WAIT_BOUND_MIN_S, WAIT_BOUND_FACTOR * pl->executed / WAIT_BOUND_RATE));
+    if (!pl->dry) rc = b.upload();
+    pl->inst.swap(b.inst);
+    if (rc == GDP_OK && !pl->dry) rc = upload_f0(pl);
+    return rc;
+}
+
 
 
 // ---- audit of a laid-out plan (gdp_debug_check_layout) -----------------------------------------------
@@ -1624,17 +1763,24 @@ int create(int32_t n, const gdp_problem *const *p, gdp_plan *pl, bool force_mark
 //   fused launches: counters cnt + (instance * max_L + layer) * max_ntile + tile;
 //   epilogue: H + (L % nbuf) * hstride + roff[L][s] + v0 with v0 in [0, V), the argmin table
 //     M + (l * S + s) * ldm + v, v in [0, V), strategy lists res + res_off + [0, L).
-int audit(const gdp_plan *pl, const gdp_problem *const *p)
+// The audit derives every bound on its own, from the plan's shapes and the caller's arrays, and compares it
+// with what the builder wrote into the tables: sharing the builder's arithmetic would check nothing.
+int audit_bad(const char *what, long long a, long long b, long long c)
 {
     char buf[256];
-    auto bad = [&](const char *what, long long a, long long b, long long c) {
-        snprintf(buf, sizeof buf, "layout audit: %s (%lld, %lld, %lld)", what, a, b, c);
-        return fail(GDP_E_HIP, buf);
-    };
-    const char *stage = pl->stage.data();
-    if (pl->stage.size() < pl->small_bytes) return bad("host copy of the tables is short", (long long)pl->stage.size(), (long long)pl->small_bytes, 0);
-    const uintptr_t base = reinterpret_cast<uintptr_t>(pl->dbase);
-    auto off_of = [&](const void *q) { return (long long)(reinterpret_cast<uintptr_t>(q) - base); };
+    snprintf(buf, sizeof buf, "layout audit: %s (%lld, %lld, %lld)", what, a, b, c);
+    return fail(GDP_E_HIP, buf);
+}
+
+long long audit_off(const gdp_plan *pl, const void *q)
+{
+    return (long long)(reinterpret_cast<uintptr_t>(q) - reinterpret_cast<uintptr_t>(pl->dbase));
+}
+
+// The sub-allocations lie inside the allocation and do not overlap.
+int audit_sub_allocations(const gdp_plan *pl)
+{
+    auto bad = audit_bad;
     // sub-allocations: inside the allocation and disjoint
     struct Span { size_t lo, hi; };
     std::vector<Span> spans;
@@ -1674,6 +1820,15 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
         if (spans[i].hi > pl->dbytes) return bad("sub-allocation beyond the allocation", (long long)spans[i].lo, (long long)spans[i].hi, (long long)pl->dbytes);
         if (i && spans[i].lo < spans[i - 1].hi) return bad("sub-allocations overlap", (long long)spans[i - 1].lo, (long long)spans[i - 1].hi, (long long)spans[i].lo);
     }
+    return GDP_OK;
+}
+
+// Instance records, row offsets, matrix indices and key records.
+int audit_instances(const gdp_plan *pl, const gdp_problem *const *p)
+{
+    auto bad = audit_bad;
+    auto off_of = [&](const void *q) { return audit_off(pl, q); };
+    const char *stage = pl->stage.data();
     const GdpDevInst *di = reinterpret_cast<const GdpDevInst *>(stage + pl->off_insts);
     const GdpDevKey *dk = reinterpret_cast<const GdpDevKey *>(stage + pl->off_keys);
     for (int i = 0; i < pl->n; ++i) {
@@ -1715,6 +1870,15 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
             if (key.other_mem < 0) return bad("start row above the table", i, k, (long long)key.other_mem);
         }
     }
+    return GDP_OK;
+}
+
+// Layer records, bands, and the grids of the three launch schemes.
+int audit_groups(const gdp_plan *pl, const gdp_problem *const *p)
+{
+    auto bad = audit_bad;
+    auto off_of = [&](const void *q) { return audit_off(pl, q); };
+    const char *stage = pl->stage.data();
     for (const Group &g : pl->groups) {
         const GdpDevLayer *lay = reinterpret_cast<const GdpDevLayer *>(stage + g.off_lay);
         const int tile_rows = 64 * GDP_VARIANTS[g.variant].r;
@@ -1810,6 +1974,16 @@ int audit(const gdp_plan *pl, const gdp_problem *const *p)
             }
     }
     return GDP_OK;
+}
+
+int audit(const gdp_plan *pl, const gdp_problem *const *p)
+{
+    if (pl->stage.size() < pl->small_bytes)
+        return audit_bad("host copy of the tables is short", (long long)pl->stage.size(), (long long)pl->small_bytes, 0);
+    int rc = audit_sub_allocations(pl);
+    if (rc == GDP_OK) rc = audit_instances(pl, p);
+    if (rc == GDP_OK) rc = audit_groups(pl, p);
+    return rc;
 }
 
 int run(gdp_plan *pl, int32_t mode, gdp_timing *t);
