@@ -131,14 +131,29 @@ def get_real_chunk(local_bsz, chunk):
     return len(chunk_like_torch(int(local_bsz), int(chunk)))
 
 
+def sum_like_numpy(values):
+    """``np.sum`` of a short list of numbers, bit for bit, without the cost of turning it into an array
+    (a sweep makes tens of thousands of such sums, a few microseconds each).  Up to seven elements numpy adds
+    them from left to right; from eight on it adds in blocks, and the list goes through numpy itself."""
+    n = len(values)
+    if n > 7:
+        return np.add.reduce(values)
+    if n == 0:
+        return np.float64(0.0)
+    acc = 0                      # numpy starts from the identity: a lone -0.0 comes out as +0.0
+    for x in values:
+        acc = acc + x
+    return acc if isinstance(acc, np.generic) else (np.int64(acc) if isinstance(acc, int) else np.float64(acc))
+
+
 def get_time_cost_all_stages(layer_timecosts, pp_stage_division):
     """Sum of the layers' times per pipeline stage (cost_model.py:687-693)."""
-    assert np.sum(pp_stage_division) == len(layer_timecosts)
+    assert sum(int(x) for x in pp_stage_division) == len(layer_timecosts)
     out, first = [], 0
-    for stage in range(len(pp_stage_division)):
-        first = int(np.sum(pp_stage_division[:stage]))
-        last = int(np.sum(pp_stage_division[:stage + 1]))
-        out.append(np.sum(layer_timecosts[first:last]))
+    for count in pp_stage_division:
+        last = first + int(count)
+        out.append(sum_like_numpy(layer_timecosts[first:last]))
+        first = last
     return out
 
 
@@ -888,13 +903,13 @@ def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_arg
     for i in range(len(other_time_cost)):
         stage_compute[i] += other_time_cost[i]
 
-    result = np.sum(stage_compute) + stage_compute[-1] * (max_chunk - 1)
+    result = sum_like_numpy(stage_compute) + stage_compute[-1] * (max_chunk - 1)
     ramp = min(pp_deg - 1, max_chunk - 1) * stage_compute[0]
-    tail = np.sum(stage_compute[1:])
+    tail = sum_like_numpy(stage_compute[1:])
     result = max(result,
                  max(ramp * 1 / 3, tail * 1 / 3) + max(ramp * 2 / 3, tail * 2 / 3)
                  + stage_compute[0] * max(0, max_chunk + 1 - pp_deg))
-    exposed = [stage_full[i] - np.sum(stage_compute[:i + 1]) for i in range(pp_deg)]
+    exposed = [stage_full[i] - sum_like_numpy(stage_compute[:i + 1]) for i in range(pp_deg)]
     reduce_time = np.max(exposed)
     result += reduce_time if reduce_time > 0 else 0
     if return_stage_cost:

@@ -237,3 +237,21 @@ def test_array_forms_decline_what_they_do_not_cover():
         M.time_cost_rows([[1, 2, 4, {'fsdp': 0}]], 64, **a)
     with pytest.raises(M.NotVectorisable):
         M.time_cost_rows([], 64, **a)
+
+
+def test_sum_like_numpy_is_numpy_sum_bit_for_bit():
+    """Short lists are added without numpy (a sweep makes tens of thousands of such sums); the result must be
+    what ``np.sum`` gives, in value, bits and type, for every length on either side of the switch to numpy."""
+    import random
+    from galvatron_dp.cost_models import sum_like_numpy
+    rng = random.Random(5)
+    for n in range(0, 13):
+        for _ in range(300):
+            xs = [rng.choice([1.0, -1.0]) * rng.random() * 10 ** rng.randint(-8, 16) for _ in range(n)]
+            if n and rng.random() < 0.3:
+                xs = [np.float64(x) for x in xs]
+            got, want = sum_like_numpy(xs), np.sum(xs)
+            assert np.float64(got).tobytes() == np.float64(want).tobytes() and type(got) is type(want), (xs, got, want)
+    assert sum_like_numpy([np.float64(-0.0)]).tobytes() == np.sum([np.float64(-0.0)]).tobytes()
+    assert sum_like_numpy([3, 4, 5]) == 12 and type(sum_like_numpy([3, 4, 5])) is type(np.sum([3, 4, 5]))
+    assert sum_like_numpy([1e16, 1.0, 1.0]) == (1e16 + 1.0) + 1.0
