@@ -850,11 +850,14 @@ class OtherTimeCostModel:
 # ---- pipeline -----------------------------------------------------------------------------------------
 def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_args_list, parallel_args_list,
                        profile_model_args_list, profile_hardware_args_list, strategies, partition, chunks, bsz, min_tp,
-                       other_time_cost, logger=None, return_stage_cost=False):
+                       other_time_cost, logger=None, return_stage_cost=False, cache=None):
     """Time of one iteration of a pipeline whose layers run the given strategies, split into stages
     by ``partition`` (cost_model.py:695-767): steady state = every stage's computation once plus
     (micro-batches - 1) times the last stage's, bounded below by the 1F1B warm-up / cool-down
-    estimate, plus the gradient synchronisation that is not hidden."""
+    estimate, plus the gradient synchronisation that is not hidden.
+    ``cache`` (no counterpart in the reference): a dict a caller keeps across calls -- a sweep asks for the
+    time of the same (layer type, strategy, micro-batch size) hundreds of times.  Entries are keyed by the
+    identity of the objects involved and keep those objects alive, so that an identity is never reused."""
     if strategies is None:
         return ([np.inf] * len(partition), np.inf) if return_stage_cost else np.inf
     type_of_layer = []
@@ -871,13 +874,31 @@ def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_arg
         max_chunk = chunks
     pp_deg = len(partition)
 
-    names = [form_strategy(s) for s in strategies]
-    texts = list(set(names))
+    if cache is None:
+        names = [form_strategy(s) for s in strategies]
+    else:
+        names = []
+        for s in strategies:
+            hit = cache.get(("form", id(s)))
+            if hit is None:
+                hit = cache[("form", id(s))] = (form_strategy(s), s)
+            names.append(hit[0])
+    all_texts = list(set(names))
     full, compute_only = {}, {}
     for t in range(len(layer_num_list)):
         common = dict(model_args=model_args_list[t], train_args=train_args_list[t], parallel_args=parallel_args_list[t],
                       profile_model_args=profile_model_args_list[t],
                       profile_hardware_args=profile_hardware_args_list[t])
+        texts = all_texts
+        if cache is not None:
+            base = ("ptime", id(timecostmodel), bsz_per_chunk[t]) + tuple(id(v) for v in common.values())
+            texts = []
+            for text in all_texts:
+                hit = cache.get(base + (text,))
+                if hit is None:
+                    texts.append(text)
+                else:
+                    full[t, text], compute_only[t, text] = hit[0], hit[1]
         rows = None
         # this package's own model: all strategies at once -- where there are enough of them for one array
         # evaluation (some sixty array operations) to be cheaper than an object per strategy
@@ -895,6 +916,9 @@ def pipeline_costmodel(timecostmodel, layer_num_list, model_args_list, train_arg
             full[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], logger=logger, **common).gen_result()
             compute_only[t, text] = timecostmodel(strategy_str2list(text), bsz_per_chunk[t], no_comm=True, logger=logger,
                                                   **common).gen_result()
+        if cache is not None:
+            for text in texts:
+                cache[base + (text,)] = (full[t, text], compute_only[t, text], timecostmodel, tuple(common.values()))
     per_layer_full = [full[type_of_layer[i], name] for i, name in enumerate(names)]
     per_layer_compute = [compute_only[type_of_layer[i], name] for i, name in enumerate(names)]
     stage_full = get_time_cost_all_stages(per_layer_full, partition)

@@ -508,10 +508,13 @@ class DpOnModel:
         flat = []
         for r in per_stage_res:
             flat += r
+        extra = {}
+        if self.row_cache is not None and self.pipeline_costmodel is cost_models.pipeline_costmodel:
+            extra["cache"] = self.row_cache       # this package's own model: per-strategy times kept across the sweep
         return self.pipeline_costmodel(self.timecost_model, self.layer_num, self.model_args_list, self.train_args_list,
                                        self.parallel_args_list, self.profile_model_args_list,
                                        self.profile_hardware_args_list, flat, P.pp_stage_list, P.chunks, P.bsz,
-                                       P.min_tp, P.other_time_cost[1][k], self.logger)
+                                       P.min_tp, P.other_time_cost[1][k], self.logger, **extra)
 
     def _finish(self, P, fits):
         pp_deg = P.pp_deg
