@@ -79,11 +79,11 @@ PEAK_HBM_GBS = 8000.0
 # bench line carries it only while both still match, null otherwise.
 MEASURED_TRAFFIC = {
     # workload (+ mode): (bytes per launch, kernel sources hash, register tile "TSxR", profile)
-    "cfg2": (12.131e9, "d18d9eb06eca2ae1", "16x1", "profiles/gdp_relax_fused_kernel_cfg2.txt"),                 # algorithmic 10.737e9
-    "cfg2+row_skipping": (7.655e9, "d18d9eb06eca2ae1", "16x1", "profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt"),
-    "cfg2+mark_table": (12.208e9, "d18d9eb06eca2ae1", "8x2", "profiles/gdp_relax_fused_kernel_cfg2_mark_table.txt"),  # algorithmic 11.409e9
-    "cfg3": (45.75e9, "d18d9eb06eca2ae1", "15x3", "profiles/gdp_relax_fused_kernel_cfg3.txt"),   # algorithmic 44.3e9; average of the 4 launches of a solve
-    "cfg4": (17.620e9, "d18d9eb06eca2ae1", "15x3", "profiles/gdp_relax_fused_kernel_cfg4.txt"),                 # algorithmic 17.716e9
+    "cfg2": (12.131e9, "5abdfea757d76060", "16x1", "profiles/gdp_relax_fused_kernel_cfg2.txt"),                 # algorithmic 10.737e9
+    "cfg2+row_skipping": (7.657e9, "5abdfea757d76060", "16x1", "profiles/gdp_relax_fused_kernel_cfg2_row_skipping.txt"),
+    "cfg2+mark_table": (12.210e9, "5abdfea757d76060", "8x2", "profiles/gdp_relax_fused_kernel_cfg2_mark_table.txt"),  # algorithmic 11.409e9
+    "cfg3": (45.78e9, "5abdfea757d76060", "15x3", "profiles/gdp_relax_fused_kernel_cfg3.txt"),   # algorithmic 44.3e9; average of the 4 launches of a solve
+    "cfg4": (17.615e9, "5abdfea757d76060", "15x3", "profiles/gdp_relax_fused_kernel_cfg4.txt"),                 # algorithmic 17.716e9
 }
 KERNEL_SOURCES = ("hetu-galvatron_amd/csrc/gdp_kernels.hip", "hetu-galvatron_amd/csrc/gdp_kernels.h")
 GOLDEN = os.path.join(ROOT, "tests", "golden", "dp_core_golden.json")

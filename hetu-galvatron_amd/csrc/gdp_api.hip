@@ -430,7 +430,8 @@ void share_equal_matrices(const gdp_problem *q, HostInst &h)
 }
 
 struct Group {  // instances with the same S, sorted by L descending
-    int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt;
+    int first, count, SP, S, max_L, max_ntile, variant, ntb, nbt;   // ntb: wave tasks per tile (with the parts of split tasks)
+    int split = 1;            // fused launches: waves that share the source strategies of a task (1, or 2: see relax_task)
     int xcd_group = 1;        // consecutive block tasks handed to one XCD (whole tiles)
     int slots = 0;            // workgroups per XCD, instance and layer of a fused launch
     int64_t max_ld;
@@ -1069,11 +1070,30 @@ int PlanBuilder::form_groups()
         const int tile_rows = 64 * best_r;
         g.SP = ntb * ts;
         g.ntb = ntb;
+        // A group whose layers hold no more wave tasks than the device has wave slots (one instance of middling
+        // size) is short of waves, not of work per wave: the sources of a task then go on two waves -- twice the
+        // waves, each half as long, so that the start of one task (a chain of dependent loads) lies behind the
+        // arithmetic of another.  Measured, relaxation time per solve, one wave -> two, every cell / with row
+        // skipping (ms): L=32 S=44 V=65536 0.441 -> 0.398 / 0.431 -> 0.386; L=28 S=40 V=65536 0.366 -> 0.322 /
+        // 0.53 -> 0.30; L=16 S=88 V=32768 0.345 -> 0.310 / 0.319 -> 0.281; L=48 S=36 V=65536 0.573 -> 0.525 /
+        // 0.80 -> 0.45; L=24 S=22 V=131072 0.280 -> 0.262 / 0.307 -> 0.243.  Not with the 16-wide tile (its
+        // exchange buffer of 32 KB holds a CU to five workgroups: L=16 S=64 V=65536 0.339 -> 0.351), and not where
+        // a layer fills the slots anyway (L=32 S=44 V=131072 0.709 -> 0.807).  GALVATRON_DP_SPLIT=1|2 overrides.
+        // (Not the narrowest tile either: plans that get it run as flow launches or with the latency variant, which
+        // split their sources in their own way and pad SU for that.)
+        if (!pl->keep_marks && best_r == GDP_SPLIT_R && ts != GDP_LAT_TS) {
+            int64_t tasks = 0;
+            for (int k = i; k < j; ++k) tasks += ((int64_t)inst[(size_t)k].V + tile_rows - 1) / tile_rows * ntb;
+            if (g.S >= 16 && ts <= 15 && tasks <= wave_slots) g.split = 2;
+            if (const char *e = getenv("GALVATRON_DP_SPLIT")) g.split = atoi(e) == 2 ? 2 : 1;
+        }
+        g.ntb = ntb * g.split;
         g.max_L = 0; g.max_ntile = 0; g.max_ld = 0;
         for (int k = i; k < j; ++k) {
             HostInst &h = inst[(size_t)k];
             h.variant = g.variant;
             h.SP = g.SP;
+            if (g.split > 1) h.SU = (int)align_up((size_t)h.S, (size_t)GDP_SRC_UNROLL * g.split);
             h.ntile = (h.V + tile_rows - 1) / tile_rows;
             h.ldm = (int64_t)align_up((size_t)h.ntile * tile_rows, 256);
             h.ld = h.P + h.ldm;
@@ -1669,6 +1689,9 @@ void PlanBuilder::build_group_tables()
             seg.lds_bytes = 0;
             if (per_cu < 8 && pl->lds_per_cu >= 65536 && !pl->no_occupancy_cap)
                 seg.lds_bytes = (unsigned)std::min<size_t>(pl->lds_per_cu / (size_t)per_cu - 1024, 65536 - 1024);
+            // (split tasks exchange their partial minima through static LDS, which counts towards the same limit)
+            const unsigned xch = (unsigned)GDP_SPLIT_LDS_BYTES(GDP_VARIANTS[g.variant].ts);
+            if (g.split > 1) seg.lds_bytes = seg.lds_bytes > xch ? seg.lds_bytes - xch : 0u;
         }
     }
 }
@@ -1882,7 +1905,13 @@ int audit_groups(const gdp_plan *pl, const gdp_problem *const *p)
     for (const Group &g : pl->groups) {
         const GdpDevLayer *lay = reinterpret_cast<const GdpDevLayer *>(stage + g.off_lay);
         const int tile_rows = 64 * GDP_VARIANTS[g.variant].r;
-        if (g.ntb * GDP_VARIANTS[g.variant].ts != g.SP) return bad("target blocks of a group", g.ntb, g.SP, 0);
+        if (g.split < 1 || g.ntb % g.split || g.ntb / g.split * GDP_VARIANTS[g.variant].ts != g.SP)
+            return bad("target blocks of a group", g.ntb, g.SP, g.split);
+        if (g.split > 1)
+            for (int k = 0; k < g.count; ++k)
+                if (pl->inst[(size_t)(g.first + k)].SU % (GDP_SRC_UNROLL * g.split) || pl->keep_marks ||
+                    GDP_VARIANTS[g.variant].r != GDP_SPLIT_R)
+                    return bad("sources of a split task", k, pl->inst[(size_t)(g.first + k)].SU, g.split);
         if (off_of(g.sched.lay) != (long long)g.off_lay || off_of(g.sched.cnt) != (long long)g.off_cnt ||
             off_of(g.sched.n_active) != (long long)g.off_active || off_of(g.sched.abort_flag) != (long long)pl->off_abort ||
             g.sched.max_L != g.max_L || g.sched.max_ntile != g.max_ntile)
@@ -2058,7 +2087,7 @@ int run_enqueue(gdp_plan *pl, int32_t mode)
                 GdpSched sched = g.sched;
                 sched.spin_limit = wait_polls(POLL_S_FUSED);
                 sched.debug_stall = pl->debug_stall ? 1 : 0;
-                GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks,
+                GDP_HIP(gdp_launch_relax_fused(g.variant, pl->keep_marks, g.split,
                                                sched, grid_x,
                                                seg.first, seg.layers, seg.lds_bytes, pl->stream));
                 if (mode >= 2) GDP_HIP(hipEventRecord(pl->ev_relax[2 * li + 1], pl->stream));
@@ -2157,6 +2186,7 @@ int run_finish(gdp_plan *pl, int32_t mode, gdp_timing *t)
             t->tile_r = GDP_VARIANTS[g0.variant].r;
             t->chunk = (pl->fused && g0.chunk < g0.count) ? g0.chunk : 0;
             t->latency_variant = pl->fused || (!pl->run_flow && !g0.lat_ok) ? 0 : g0.latency;
+            t->fused_split = pl->fused ? g0.split : 1;
         }
         t->keep_marks = pl->keep_marks ? 1 : 0;
         if (mode >= 1) GDP_HIP(hipEventElapsedTime(&t->total_ms, pl->ev_begin, pl->ev_end));

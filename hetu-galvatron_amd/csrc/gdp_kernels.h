@@ -151,7 +151,12 @@ hipError_t gdp_launch_relax(int variant, bool marks, int latency, const GdpDevLa
 // layers): a block waits on per-tile completion counters instead of on a kernel boundary.
 // lds_bytes: dynamic LDS per workgroup, unused by the kernel; it limits how many workgroups a CU holds.
 // With sched->rows set, layer0 is the first entry of that table and `layers` the number of entries.
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched, int grid_blocks, int layer0,
+// split: 1, or 2 -- the source strategies of a wave task on two waves of a workgroup (costs only, register
+// tiles of 64 rows, GDP_SPLIT_R == 1; the layers' SU is then a multiple of 2 * GDP_SRC_UNROLL, sched.ntb counts
+// both parts of every task, and every workgroup also takes GDP_SPLIT_LDS_BYTES(ts) of static LDS).
+#define GDP_SPLIT_R 1
+#define GDP_SPLIT_LDS_BYTES(ts) (GDP_WAVES_PER_BLOCK * GDP_SPLIT_R * (ts) * 64 * 8)
+hipError_t gdp_launch_relax_fused(int variant, bool marks, int split, const GdpSched &sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream);
 // (sources per wave, waves per task) of the flow kernels that are built
 #define GDP_FOR_EACH_FLOW(X) \

@@ -514,15 +514,23 @@ __device__ __forceinline__ void relax_task_flow(const FlowHead &H, unsigned tile
 // it a relaxation is one addition and one minimum (intra is added once per cell, see the top of this
 // file); the backtrack then recomputes the argmin of the few cells on its path from the cost
 // buffers, all of which are kept in that mode.
-template <int TS, int R, bool PUBLISH, bool ARG>
-__device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, unsigned tb, unsigned lane)
+// K > 1 (costs only): the source strategies of a task are split over K waves of the workgroup (vtb =
+// target block * K + part; part p takes sources [p * SU / K, (p + 1) * SU / K), SU being a multiple of K times
+// the sources per trip) -- for launches whose layers hold too few wave tasks to keep the device's wave slots
+// filled: twice the waves, each half as long.  The partial minima meet in LDS; the minimum of the parts is
+// the minimum over all sources exactly (min is associative and commutative), and the wave of part j % K adds
+// intra to column j and stores it.  Every part counts as a finished wave task of its tile.
+template <int TS, int R, bool PUBLISH, bool ARG, int K = 1>
+__device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, unsigned vtb, unsigned lane)
 {
-    const int SU = uload(&Y->SU);
+    static_assert(K == 1 || (!ARG && GDP_WAVES_PER_BLOCK % K == 0), "parts of one task share a workgroup; costs only");
+    const unsigned tb = vtb / K, part = vtb % K;
+    const int SU = uload(&Y->SU) / K;
     const int SP = uload(&Y->SP);
     const double *src = uload(&Y->src);
-    const int64_t *ro = uload(&Y->ro);
+    const int64_t *ro = uload(&Y->ro) + part * SU;
     const int s0 = tb * TS;
-    const double *it = uload(&Y->it) + s0;
+    const double *it = uload(&Y->it) + s0 + (int64_t)part * SU * SP;
     const double *ia = uload(&Y->ia) + s0;
     const int64_t u0 = (int64_t)tile * (64 * R);
 
@@ -611,6 +619,29 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
     // made before the loop.)
     const GdpDevLayer *Z = Y;
     asm volatile("" : "+s"(Z));
+    bool mine[TS];
+#pragma unroll
+    for (int j = 0; j < TS; ++j) mine[j] = true;
+    if constexpr (K > 1) {
+        __shared__ double xch[GDP_WAVES_PER_BLOCK][R][TS][64];
+        const unsigned wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < TS; ++j) xch[wv][r][j][lane] = best[r][j];
+        __syncthreads();   // waves of the workgroup that had no task have ended and are not waited for
+        const unsigned w0 = wv - part;   // the task's first wave
+#pragma unroll
+        for (int j = 0; j < TS; ++j) {
+            mine[j] = (unsigned)(j % K) == part;
+            if (mine[j]) {
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int pp = 0; pp < K; ++pp) best[r][j] = min_f64(best[r][j], xch[w0 + pp][r][j][lane]);
+            }
+        }
+    }
     if constexpr (!ARG) {
         const double *iz = uload(&Z->ia) + s0;
 #pragma unroll
@@ -634,6 +665,7 @@ __device__ __forceinline__ void relax_task(const GdpDevLayer *Y, unsigned tile, 
         if (j < nvalid) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
+                if (!mine[j]) continue;
                 if (PUBLISH)
                     __hip_atomic_store(drow + (lane + 64u * r), best[r][j], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
@@ -691,7 +723,7 @@ __device__ __forceinline__ void fill_task(const GdpDevLayer *Y, unsigned tile, u
 // Rows of a layer that have to be computed (tiles lo .. hi): below the band every source cell is
 // +inf (fill_task); above it no cell can lie on a path that ends at one of the requested start
 // rows, so nothing is read from there later and nothing is written.
-template <int TS, int R, bool PUBLISH, bool ARG>
+template <int TS, int R, bool PUBLISH, bool ARG, int K = 1>
 __device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, unsigned tile, unsigned tb,
                                           unsigned lane)
 {
@@ -700,7 +732,7 @@ __device__ __forceinline__ void tile_task(const GdpDevLayer *Y, int lo, int hi, 
         // costs only: every layer has a buffer of its own, and these rows were filled when the plan was made
         if constexpr (ARG) fill_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
     } else {
-        relax_task<TS, R, PUBLISH, ARG>(Y, tile, tb, lane);
+        relax_task<TS, R, PUBLISH, ARG, K>(Y, tile, tb, lane);   // (K > 1: tb counts the parts of the split tasks too)
     }
 }
 
@@ -822,7 +854,9 @@ __device__ __forceinline__ bool wait_tiles(const int32_t *cnt, int lo, int hi, i
 //    before its counter is full, and the caches are invalidated when the launch begins.
 //
 // Share of an XCD: of every instance, every eighth group of block tasks (see below).
-template <int TS, int R, bool ARG>
+// K > 1: the sources of a task are split over K waves (see relax_task); Q.ntb then counts the parts, so that
+// a tile is finished when ntb wave tasks have counted themselves.
+template <int TS, int R, bool ARG, int K = 1>
 __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK) void gdp_relax_fused_kernel(
     const GdpSched Q, int layer0)
 {
@@ -894,7 +928,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
         const unsigned qq = bt * GDP_WAVES_PER_BLOCK + wave;
         const unsigned tl = qq / ntb, tbb = qq - tl * ntb;
         const int64_t *ro_ = uload(&Y->ro);
-        const double *it_ = uload(&Y->it) + tbb * TS;
+        const double *it_ = uload(&Y->it) + (tbb / K) * TS;
         pf_o = uload(ro_);
         pf_a = uload(it_);
         pf_b = uload(it_ + (TS - 1));
@@ -926,7 +960,7 @@ __global__ __launch_bounds__(64 * GDP_WAVES_PER_BLOCK, 16 / GDP_WAVES_PER_BLOCK)
     const unsigned tb = q - tile * ntb;
     if (tile >= (unsigned)ntile) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");    // keeps the tile's loads after the wait
-    tile_task<TS, R, true, ARG>(Y, lo, hi, tile, tb, lane);   // with the argmin table: tiles outside the band
+    tile_task<TS, R, true, ARG, K>(Y, lo, hi, tile, tb, lane);   // with the argmin table: tiles outside the band
                                                               // are filled or skipped there and count as done
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // every write-through store acknowledged
@@ -1470,9 +1504,18 @@ static hipError_t launch_relax_v(bool marks, const GdpDevLayer *lay, int max_L, 
 }
 
 template <int TS, int R, bool MARKS_BUILT>
-static hipError_t launch_fused_v(bool marks, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
+static hipError_t launch_fused_v(bool marks, int split, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream,
                           const GdpSched &sched, int layer0)
 {
+    if (split != 1) {
+        if constexpr (R == GDP_SPLIT_R) {
+            if (split == 2 && !marks) {
+                hipLaunchKernelGGL((gdp_relax_fused_kernel<TS, R, false, 2>), grid, block, lds_bytes, stream, sched, layer0);
+                return hipGetLastError();
+            }
+        }
+        return hipErrorInvalidValue;
+    }
     if constexpr (MARKS_BUILT) {
         if (marks) {
             hipLaunchKernelGGL((gdp_relax_fused_kernel<TS, R, true>), grid, block, lds_bytes, stream, sched, layer0);
@@ -1508,12 +1551,12 @@ hipError_t gdp_launch_relax(int variant, bool marks, int latency, const GdpDevLa
 #undef X
 }
 
-hipError_t gdp_launch_relax_fused(int variant, bool marks, const GdpSched &sched, int grid_blocks, int layer0,
+hipError_t gdp_launch_relax_fused(int variant, bool marks, int split, const GdpSched &sched, int grid_blocks, int layer0,
                                   int layers, unsigned lds_bytes, hipStream_t stream)
 {
     dim3 grid((unsigned)grid_blocks, (unsigned)layers), block(64 * GDP_WAVES_PER_BLOCK);
 #define X(id, ts, r, m) \
-    case id: return launch_fused_v<ts, r, m>(marks, grid, block, lds_bytes, stream, sched, layer0);
+    case id: return launch_fused_v<ts, r, m>(marks, split, grid, block, lds_bytes, stream, sched, layer0);
     switch (variant) {
         GDP_FOR_EACH_VARIANT(X)
         default: return hipErrorInvalidValue;

@@ -75,7 +75,7 @@ class gdp_timing(ctypes.Structure):
                 ("fused", ctypes.c_int32), ("relaxations", ctypes.c_double), ("executed", ctypes.c_double),
                 ("relax_bytes", ctypes.c_double), ("tile_ts", ctypes.c_int32), ("tile_r", ctypes.c_int32),
                 ("keep_marks", ctypes.c_int32), ("chunk", ctypes.c_int32),
-                ("latency_variant", ctypes.c_int32), ("flow", ctypes.c_int32)]
+                ("latency_variant", ctypes.c_int32), ("flow", ctypes.c_int32), ("fused_split", ctypes.c_int32)]
 
 
 class gdp_batch_stats(ctypes.Structure):

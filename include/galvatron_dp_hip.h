@@ -120,6 +120,7 @@ typedef struct gdp_timing {
     int32_t latency_variant; /* > 0: per-layer launches use the kernel variant for launches with few waves,
                                 with the source strategies of a task on this many waves (1, 2 or 4) */
     int32_t flow;          /* 1: all layers in one launch whose tasks wait on the cost cells themselves (small plans) */
+    int32_t fused_split;   /* fused launches: waves that share the source strategies of a wave task (1 or 2)         */
 } gdp_timing;
 
 typedef struct gdp_plan gdp_plan;

@@ -30,7 +30,7 @@ def test_version_and_struct_sizes():
     assert _lib.lib().gdp_version() == 102
     assert ctypes.sizeof(_lib.gdp_problem) == 88
     assert ctypes.sizeof(_lib.gdp_result) == 40
-    assert ctypes.sizeof(_lib.gdp_timing) == 64
+    assert ctypes.sizeof(_lib.gdp_timing) == 72
 
 
 def test_validation_happens_before_any_device_work():

@@ -162,3 +162,86 @@ def test_many_threads_share_the_library():
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+SPLIT_SHAPES = [(3, 1, 64), (4, 7, 191), (5, 11, 256), (3, 12, 257), (4, 22, 512), (3, 33, 700), (6, 44, 1000), (2, 45, 130),
+                (3, 64, 333), (2, 88, 410), (2, 129, 131), (9, 23, 2048), (12, 44, 4099), (2, 300, 150)]
+
+
+@pytest.mark.parametrize("n,shape", list(enumerate(SPLIT_SHAPES)))
+def test_sources_of_a_task_split_over_two_waves(n, shape, monkeypatch):
+    """Fused launches whose layers hold few wave tasks put the source strategies of a task on two waves
+    (partial minima combined through LDS: exact, the minimum being associative).  Forced here on every shape
+    -- odd numbers of sources, fewer sources than a trip, rows that do not fill a tile, +inf, ties -- with
+    unwritten cells poisoned, against the C oracle: results and the full f array."""
+    if any(k in os.environ for k in ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R",
+                                     "GALVATRON_DP_FUSED", "GALVATRON_DP_SPLIT")):
+        pytest.skip("the environment presets the layout")
+    L, S, V = shape
+    monkeypatch.setenv("GALVATRON_DP_TILE_TS", "11")
+    monkeypatch.setenv("GALVATRON_DP_TILE_R", "1")
+    monkeypatch.setenv("GALVATRON_DP_SPLIT", "2")
+    for variant in range(3):
+        rng = np.random.Generator(np.random.PCG64([78, n, variant]))
+        inst = W.random_instance(rng, L, S, V, integer_costs=variant == 1, mem_hi=[max(1, V // (L + 1)), max(1, V // 2), V + 3][variant],
+                                 per_layer_inter=bool(variant % 2), inf_frac=0.2 if variant == 2 else 0.0,
+                                 over_frac=0.1 if variant == 2 else 0.0, n_keys=3)
+        keys = sorted(inst.other_mem)
+        want = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, keep=True)
+        for compute_all in (False, True):
+            prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                                [inst.other_time[k] for k in keys], inter_index=inst.inter_index, export_f=compute_all,
+                                launch="fused", compute_all=compute_all)
+            with _lib.Plan([prob]) as plan:
+                plan.set_option(_lib.GDP_OPT_POISON, 1)
+                for _ in range(2):
+                    t = plan.run(1)
+                    assert t.fused == 1 and t.fused_split == 2 and t.tile_ts == 11 and t.tile_r == 1
+                    plan.fetch()
+                    got = ({k: prob.total[i] for i, k in enumerate(keys)},
+                           {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+                           {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+                    H.assert_same_results(got, want[:3], f"split, shape {shape} variant {variant} compute_all={compute_all}")
+                    if compute_all:
+                        assert prob.f_out.tobytes() == want[3].tobytes()
+            # the same plan given up (host-forced) repeats the solve with one launch per layer, tasks whole again
+            with _lib.Plan([prob]) as plan:
+                plan.set_option(_lib.GDP_OPT_SPIN_LIMIT, 1)
+                plan.run()
+                plan.fetch()
+                got = ({k: prob.total[i] for i, k in enumerate(keys)},
+                       {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+                       {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+                H.assert_same_results(got, want[:3], f"split plan after a give-up, shape {shape} variant {variant}")
+
+
+def test_split_tasks_in_a_batch_of_different_depths(monkeypatch):
+    """Several instances of one strategy count, different depths and budgets, in one plan whose fused
+    launches split their tasks' sources (one launch per run of layers with the same set of instances)."""
+    if any(k in os.environ for k in ("GALVATRON_DP_KEEP_MARKS", "GALVATRON_DP_TILE_TS", "GALVATRON_DP_TILE_R",
+                                     "GALVATRON_DP_FUSED", "GALVATRON_DP_SPLIT")):
+        pytest.skip("the environment presets the layout")
+    monkeypatch.setenv("GALVATRON_DP_TILE_TS", "11")
+    monkeypatch.setenv("GALVATRON_DP_TILE_R", "1")
+    monkeypatch.setenv("GALVATRON_DP_SPLIT", "2")
+    rng = np.random.Generator(np.random.PCG64(4242))
+    insts = [W.random_instance(rng, L, 44, V, mem_hi=max(1, V // (L + 1)), integer_costs=bool(n % 2), per_layer_inter=bool(n % 3),
+                               inf_frac=0.1 * (n % 2), n_keys=3)
+             for n, (L, V) in enumerate([(9, 3000), (4, 700), (9, 5000), (2, 129), (6, 2048), (1, 64)])]
+    probs = []
+    for inst in insts:
+        keys = sorted(inst.other_mem)
+        probs.append(_lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                                  [inst.other_time[k] for k in keys], inter_index=inst.inter_index, launch="fused"))
+    with _lib.Plan(probs) as plan:
+        plan.set_option(_lib.GDP_OPT_POISON, 1)
+        t = plan.run(1)
+        assert t.fused == 1 and t.fused_split == 2
+        plan.fetch()
+    for n, (inst, prob) in enumerate(zip(insts, probs)):
+        keys = sorted(inst.other_mem)
+        want = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time)
+        got = ({k: prob.total[i] for i, k in enumerate(keys)},
+               {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
+               {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
+        H.assert_same_results(got, want, f"instance {n}")
