@@ -195,6 +195,17 @@ def galvatron_like() -> Instance:
 CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4}
 
 
+def zero_memory_tiny_budget(seed: int, L: int, S: int, V: int) -> Instance:
+    """Memory costs of 0 and 1 under a budget of a few bins: the in-place update then chains cells of one
+    layer (csrc/dp_core.cpp:58-73), and the reference's walk back, which does not know that, can arrive at
+    a negative row (csrc/dp_core.cpp:105-113)."""
+    rng = np.random.Generator(np.random.PCG64([8, seed, L, S, V]))
+    inst = random_instance(rng, L, S, V, mem_lo=0, mem_hi=max(1, V // (L + 1)), n_keys=4)
+    inst.other_mem = {k: int(rng.integers(0, V)) for k in inst.other_mem}
+    inst.other_mem[min(inst.other_mem)] = 0
+    return inst
+
+
 def with_initial_costs(inst: Instance, rng, *, integer: bool = False, inf_frac: float = 0.0) -> Instance:
     """``inst`` with a non-zero ``_f`` on entry: the reference relaxes in place from whatever the caller's
     array holds (csrc/dp_core.cpp:46-47,67).  Finite entries (small integers with ``integer``, so that

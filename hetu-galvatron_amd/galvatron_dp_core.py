@@ -17,7 +17,8 @@ device in a compact form, and copying L*V*S int32 back per call would dominate t
 Inputs on which the reference's result depends on evaluation order or is undefined raise
 ``ValueError`` instead of computing something: NaN / -inf costs (also in ``_f``), a -0.0 in ``_f``,
 negative memory costs, a negative ``other_mem_cost`` (start row above the table).  A memory cost of 0 is computed with the reference's
-in-place order (csrc/dp_core.cpp:58-73).
+in-place order (csrc/dp_core.cpp:58-73); where the reference's walk back would then index its argmin table
+with a negative row (undefined behaviour, csrc/dp_core.cpp:105-113) the key comes back as infeasible.
 """
 from __future__ import annotations
 

@@ -71,7 +71,11 @@ typedef struct gdp_problem {
     const int32_t *mem;         /* [L][S]  memory cost in bins, >= 0.  An entry of 0 is computed with the reference's
                                             in-place semantics (such a cell reads its own row, where lower strategies
                                             already hold the layer's values: csrc/dp_core.cpp:58-73); a plan with such
-                                            entries runs one launch per layer                                   */
+                                            entries runs one launch per layer.  The reference's walk back does not
+                                            know of those same-layer candidates and can then arrive at a negative
+                                            row, with which it indexes its argmin table (csrc/dp_core.cpp:105-113:
+                                            undefined behaviour); the library stops there and reports the key as
+                                            infeasible (total +inf, remaining -1)                              */
     const double *intra;        /* [L][S]                                                          */
     const double *inter;        /* [n_inter][S][S], row = source strategy, column = target        */
     const int32_t *inter_index; /* [L] layer -> matrix in `inter`; NULL means n_inter == L, identity */

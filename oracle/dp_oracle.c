@@ -85,7 +85,17 @@ void dp_oracle_relax(int L, int V, int S, const int32_t *mem,
 /* Epilogue for ONE key, csrc/dp_core.cpp:80-116.  Callers iterate keys in
  * ascending order.  res[L] is written only when the key is feasible (the
  * reference leaves the caller's -1 fill in place otherwise).
- * Exactly one of mark / mark8 must be non-NULL when L > 1. */
+ * Exactly one of mark / mark8 must be non-NULL when L > 1.
+ *
+ * With memory costs of 0 the reference's walk can leave the table: such a
+ * cell took candidates from its OWN layer (the update is in place), the walk
+ * back does not know that, follows the argmin as if it pointed into the layer
+ * before, and can arrive at a negative row, which the reference then uses in
+ * its flat index `mark[i*V*S + v*S + cur]` (:110) -- an element of an earlier
+ * layer's rows, or memory in front of the array: undefined behaviour.  This
+ * restatement forms the same flat index while it stays inside the array (so
+ * that it gives what the reference's build gives there) and stops where it
+ * would not; dp_oracle_walk_leaves_table() says whether a key is such a case. */
 void dp_oracle_epilogue(int L, int V, int S, const int32_t *mem,
                         const double *f, const int32_t *mark,
                         const int8_t *mark8, int64_t other_mem,
@@ -104,12 +114,39 @@ void dp_oracle_epilogue(int L, int V, int S, const int32_t *mem,
     res[L - 1] = idx;
     for (int i = L - 1; i > 0; --i) {
         int cur = idx;
-        size_t cell = ((size_t)i * V + v) * S + idx;
+        int64_t row = (int64_t)i * V + v;           /* v may be negative here: see above */
+        if (row < 0) { *remaining = INT32_MIN; return; }
+        size_t cell = (size_t)row * S + idx;
         idx = mark ? mark[cell] : (int)mark8[cell];
+        if (idx < 0 || idx >= S) { *remaining = INT32_MIN; return; }   /* a -1 read from an earlier layer's rows */
         v -= mem[(size_t)i * S + cur];
         res[i - 1] = idx;
     }
     *remaining = v - mem[idx];
+}
+
+/* 1 when the reference's walk back for this key indexes mark with a negative
+ * row (undefined behaviour in the reference, see above), else 0. */
+int dp_oracle_walk_leaves_table(int L, int V, int S, const int32_t *mem,
+                                const double *f, const int32_t *mark,
+                                const int8_t *mark8, int64_t other_mem)
+{
+    int64_t v0 = (int64_t)V - 1 - other_mem;
+    if (v0 < 0) return 0;
+    const double *row = f + (size_t)v0 * S;
+    int idx = 0;
+    for (int s = 1; s < S; ++s) if (row[s] < row[idx]) idx = s;
+    if (!(row[idx] < INFINITY)) return 0;
+    int64_t v = v0;
+    for (int i = L - 1; i > 0; --i) {
+        if (v < 0) return 1;
+        int cur = idx;
+        size_t cell = ((size_t)i * V + (size_t)v) * S + idx;
+        idx = mark ? mark[cell] : (int)mark8[cell];
+        if (idx < 0 || idx >= S) return 1;
+        v -= mem[(size_t)i * S + cur];
+    }
+    return 0;
 }
 
 /* Whole call: layer loop + epilogue for n_key keys (already ascending). */

@@ -42,6 +42,8 @@ def lib():
         L.dp_oracle_solve.restype = None
         L.dp_oracle_solve.argtypes = [ctypes.c_int] * 3 + [_i32p, _f64p, _f64p, _f64p, _i32p, _i8p,
                                                          ctypes.c_int, _i64p, _f64p, _f64p, _i32p, _i32p]
+        L.dp_oracle_walk_leaves_table.restype = ctypes.c_int
+        L.dp_oracle_walk_leaves_table.argtypes = [ctypes.c_int] * 3 + [_i32p, _f64p, _i32p, _i8p, ctypes.c_int64]
         L.dp_oracle_relax.restype = None
         L.dp_oracle_relax.argtypes = [ctypes.c_int] * 3 + [_i32p, _f64p, _f64p, _f64p, _i32p, _i8p]
         L.dp_oracle_coarse.restype = None
@@ -51,10 +53,13 @@ def lib():
     return _lib
 
 
-def solve(mem, intra, inter, V, other_mem, other_time, *, f0=None, mark_dtype=np.int32, keep=False):
+def solve(mem, intra, inter, V, other_mem, other_time, *, f0=None, mark_dtype=np.int32, keep=False, undefined=None):
     """Run the C restatement.  Returns ``(total, res, remaining)`` dicts keyed like
     ``other_mem`` (ascending), plus ``(f, mark)`` in the reference's layouts when
-    ``keep`` is true.  ``mark_dtype`` int32 (reference) or int8 (compact)."""
+    ``keep`` is true.  ``mark_dtype`` int32 (reference) or int8 (compact).
+    ``undefined``: a set that receives the keys for which the reference's walk back indexes its argmin table
+    with a negative row -- possible only with memory costs of 0, undefined behaviour in the reference
+    (csrc/dp_core.cpp:105-113), so their strategy list and remaining memory mean nothing."""
     mem = np.ascontiguousarray(mem, dtype=np.int32)
     intra = np.ascontiguousarray(intra, dtype=np.float64)
     inter = np.ascontiguousarray(inter, dtype=np.float64)
@@ -73,6 +78,11 @@ def solve(mem, intra, inter, V, other_mem, other_time, *, f0=None, mark_dtype=np
     lib().dp_oracle_solve(L, V, S, _ptr(mem, _i32p), _ptr(intra, _f64p), _ptr(inter, _f64p), _ptr(f, _f64p),
                           _ptr(m32, _i32p), _ptr(m8, _i8p), len(keys), _ptr(om, _i64p), _ptr(ot, _f64p),
                           _ptr(total, _f64p), _ptr(rem, _i32p), _ptr(res, _i32p))
+    if undefined is not None:
+        for i, k in enumerate(keys):
+            if lib().dp_oracle_walk_leaves_table(L, V, S, _ptr(mem, _i32p), _ptr(f, _f64p), _ptr(m32, _i32p), _ptr(m8, _i8p),
+                                                 int(om[i])):
+                undefined.add(k)
     out = ({k: float(total[i]) for i, k in enumerate(keys)},
            {k: [int(x) for x in res[i]] for i, k in enumerate(keys)},
            {k: int(rem[i]) for i, k in enumerate(keys)})

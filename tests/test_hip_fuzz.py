@@ -245,3 +245,27 @@ def test_split_tasks_in_a_batch_of_different_depths(monkeypatch):
                {k: [int(x) for x in prob.res[i]] for i, k in enumerate(keys)},
                {k: int(prob.remaining[i]) for i, k in enumerate(keys)})
         H.assert_same_results(got, want, f"instance {n}")
+
+
+@pytest.mark.parametrize("seed,shape", list(enumerate([(8, 17, 1), (12, 31, 65), (9, 8, 5), (6, 40, 64), (13, 5, 3), (10, 22, 7)])))
+def test_keys_whose_reference_walk_leaves_the_table_are_reported_infeasible(seed, shape):
+    """With memory costs of 0 and a budget of a few bins the reference's walk back can arrive at a negative
+    row and index its argmin table with it (undefined behaviour, csrc/dp_core.cpp:105-113).  The library walks
+    the same way but stops there: such a key comes back as infeasible (+inf, -1, strategy list untouched);
+    every other key equals the reference's, costs-only and with the argmin table."""
+    L, S, V = shape
+    inst = W.zero_memory_tiny_budget(seed, L, S, V)
+    undefined = set()
+    want = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time, undefined=undefined)
+    keys = sorted(inst.other_mem)
+    for keep_marks in (False, True):
+        prob = _lib.Problem(inst.mem, inst.intra, inst.inter_tables, inst.V, [inst.other_mem[k] for k in keys],
+                            [inst.other_time[k] for k in keys], inter_index=inst.inter_index, keep_marks=keep_marks)
+        _lib.solve_batch([prob])
+        for i, k in enumerate(keys):
+            if k in undefined:
+                assert prob.total[i] == np.inf and prob.remaining[i] == -1 and (prob.res[i] == -1).all(), (k, prob.total[i])
+            else:
+                assert np.float64(prob.total[i]).tobytes() == np.float64(want[0][k]).tobytes(), (k, prob.total[i], want[0][k])
+                assert int(prob.remaining[i]) == want[2][k]
+                assert want[2][k] == -1 or [int(x) for x in prob.res[i]] == want[1][k]

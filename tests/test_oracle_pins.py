@@ -251,3 +251,28 @@ def test_coarse_branch_against_the_reference_scenarios(name, monkeypatch):
     dpm = stubs.build(DpOnModel, cfg, other_timecost_model=stubs.StubOther, pipeline_costmodel=stubs.stub_pipeline_costmodel)
     assert stubs.run(dpm, cfg) == want
     assert len(seen) >= 3, "the scenario should have gone through the coarse branch for every stage"
+
+
+def test_the_reference_walk_can_leave_the_table_with_memory_costs_of_zero():
+    """A cell whose memory cost is 0 takes candidates from its own layer (the update is in place), but the
+    walk back follows its argmin as if it pointed into the layer before; under a budget of a few bins it then
+    arrives at a negative row, with which the reference indexes its argmin table (csrc/dp_core.cpp:105-113):
+    undefined behaviour.  The restatement says which keys those are, and agrees with the reference's build on
+    all the others."""
+    from galvatron_dp import workloads as W
+    flagged = 0
+    for seed, (L, S, V) in enumerate([(8, 17, 1), (12, 31, 65), (9, 8, 5), (6, 40, 64), (13, 5, 3), (10, 22, 7)]):
+        inst = W.zero_memory_tiny_budget(seed, L, S, V)
+        undefined = set()
+        total, res, rem = O.solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time,
+                                  undefined=undefined)
+        flagged += len(undefined)
+        for k in undefined:
+            assert total[k] < math.inf            # the cost itself is what the in-place update computed
+        if O.ref_available():
+            rt, rr, rm = O.ref_solve(inst.mem, inst.intra, inst.inter, inst.V, inst.other_mem, inst.other_time)
+            for k in total:
+                assert np.float64(total[k]).tobytes() == np.float64(rt[k]).tobytes()
+                if k not in undefined:
+                    assert rem[k] == rm[k] and (rm[k] == -1 or res[k] == rr[k]), (seed, k)
+    assert flagged >= 3, "the cases should include keys whose walk leaves the table"
