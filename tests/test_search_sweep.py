@@ -73,3 +73,24 @@ def test_result_file_fields():
     assert cfg["checkpoint"] == "0,1,0" and cfg["pp_division"] == "2,1" and cfg["global_bsz"] == 32
     assert cfg["chunks"] == 4 and cfg["vtp"] == 2 and cfg["embed_sdp"] == 1 and cfg["pipeline_type"] == "pipedream_flush"
     assert e.result_config(dict(min_pp_deg=-1, min_res_list=None), 32, 4, {}) is None
+
+
+def test_a_failure_while_tasks_are_prepared_leaves_the_engine_as_it_was(tmp_path):
+    """``parallelism_optimization`` works on a copy of the strategy list and hands parts of the batch to a
+    worker thread: whatever goes wrong while the tasks are prepared, the engine holds its own list again
+    afterwards and no worker is left behind (no device is needed: the failure comes before the first part)."""
+    import threading
+
+    from galvatron_dp import cost_models
+    engine = S.build(SearchEngine, cost_models, "llama_like", str(tmp_path))
+    mine = engine.strategies
+    before = threading.active_count()
+
+    def boom(*a, **k):
+        raise RuntimeError("cost model failed")
+
+    engine._task_strategies = boom
+    with pytest.raises(RuntimeError, match="cost model failed"):
+        engine.parallelism_optimization()
+    assert engine.strategies is mine
+    assert threading.active_count() == before
