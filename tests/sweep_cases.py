@@ -51,6 +51,18 @@ SWEEPS = {
     'bsz_range': dict(args=dict(min_bsz=16, max_bsz=32, bsz_scale=16, settle_chunk=2, max_tp_deg=2, sp_space='tp',
                                 global_memory_buffer=0, memory_constraint=12, disable_sdp=1),
                       layers=[(10, 4096, 1024)], params=[80.0], profile_seeds=[45]),
+    # one strategy for all layers of a stage (the coarse branch of DPAlg.fit, dynamic_programming.py:62-75)
+    'coarse': dict(args=dict(settle_bsz=32, settle_chunk=2, max_tp_deg=4, memory_constraint=8, fine_grained_mode=0),
+                   layers=[(12, 4096, 2048)], params=[96.0], profile_seeds=[46]),
+    # no pipeline cost model behind the DP, ZeRO-2 as the data-parallel default, gradients reduced synchronously
+    'flat_zero2': dict(args=dict(settle_bsz=48, max_tp_deg=4, memory_constraint=10, use_pipeline_costmodel=0,
+                                 default_dp_type='zero2', sp_space='tp'),
+                       layers=[(8, 4096, 2048)], params=[120.0], profile_seeds=[47],
+                       train=dict(async_grad_reduce=False), parallel=dict(use_zero2_for_dp=True)),
+    # no pipeline parallelism at all, two layer types, checkpointing and consecutive-tp variants off
+    'no_pp': dict(args=dict(settle_bsz=16, search_space='dp+tp', disable_ckpt=1, disable_tp_consec=1,
+                            memory_constraint=14, max_tp_deg=8),
+                  layers=[(4, 4096, 1024), (6, 4096, 2048)], params=[60.0, 110.0], profile_seeds=[48, 49]),
 }
 
 
@@ -66,9 +78,11 @@ def build(engine_cls, args_mod, name, workdir):
         prof = C.profile(np.random.Generator(np.random.PCG64([77, cfg['profile_seeds'][i]])))
         model = dict(parameter_size=cfg['params'][i], seq_length=s, hidden_size=h, layer_num=24)
         train = dict(mixed_precision=args.mixed_precision != 'fp32', async_grad_reduce=True, pytorch_context_mem=1024)
+        train.update(cfg.get('train', {}))
         parallel = dict(use_zero2_for_dp=False, disable_vtp=bool(args.disable_vtp), sequence_parallel=True,
                         sp_space=args.sp_space, pipeline_type=args.pipeline_type, optimal_chunk_func=C.chunk_func,
                         chunks=None)
+        parallel.update(cfg.get('parallel', {}))
         for lst, rec in zip(lists, C._records(args_mod, prof, model, train, parallel)):
             lst.append(rec)
     if hasattr(engine, 'set_model'):
