@@ -68,6 +68,7 @@ class SearchEngine:
         args.gpu_num = args.num_nodes * args.num_gpus_per_node
         self.memory_constraint = args.memory_constraint * 1024
         self.optimal_chunk_func = optimal_chunk_func_default
+        self.model_type = 'gpt'
         self.model_name = None
         self.path = None
         self.mem_path = None
@@ -102,6 +103,19 @@ class SearchEngine:
     def set_model_name(self, name):
         self.model_name = name
 
+    def set_model_type(self, model_type):
+        """Kept for the scripts that call it (search_engine.py:55-56); nothing in a search reads it."""
+        self.model_type = model_type
+
+    def set_microbatch_func(self, microbatch_size, max_chunk):
+        """Chunk counts from a fixed micro-batch size instead of the one each task implies
+        (search_engine.py:88-89); to be called before the cost-model records are built.  The reference
+        installs a callable of two arguments here while every call site passes four (cost_model.py:79,
+        dynamic_programming.py:224, search_engine.py:1103), so its own searches raise TypeError after this
+        call; this one takes the four arguments.  ``max_chunk`` is not used, as in the reference."""
+        self.optimal_chunk_func = lambda local_bsz, strategy, mbsz=None, min_tp=1: optimal_chunk_func_default(
+            local_bsz, strategy, microbatch_size, min_tp)
+
     def set_model_layer_configs(self, model_layer_configs):
         if model_layer_configs is None:
             return
@@ -131,6 +145,42 @@ class SearchEngine:
         self.get_profiled_model_configs()
         self.get_profiled_hardware_configs()
         self.set_cost_models()
+        self.show_search_info()
+
+    def show_search_info(self):
+        """What the search will work with, printed (search_engine.py:916-969)."""
+        args, bar = self.args, '=' * 80
+        sections = [
+            ('--- Optimization Configs ----',
+             [('Memory constraint: %d GB' % args.memory_constraint,), ('Pipeline Type:', args.pipeline_type),
+              ('Default DP Type:', args.default_dp_type), ('Mixed Precision:', args.mixed_precision), ('Search Space:',),
+              (', '.join(cost_models.form_strategy(s) for s in self.strategies or []),)]),
+            ('---- Environment Configs ----',
+             [('Allreduce Bandwidth (GB/s):', getattr(self, 'allreduce_bandwidth', None)),
+              ('Allreduce Communication Coefficient (ms/MB):', getattr(self, 'allreduce_comm_coe', None)),
+              ('P2P Bandwidth (GB/s):', getattr(self, 'p2p_bandwidth', None)),
+              ('P2P Communication Coefficient (ms/MB):', getattr(self, 'p2p_comm_coe', None)),
+              ('Overlap coefficient:', getattr(self, 'overlap_coe', None))]),
+            ('------- Model Configs -------',
+             [('Model Name:', self.model_name), ('Num layertype:', self.num_layertype), ('Layer_num:', self.layernum_list),
+              ('Hidden_size:', self.hiddensize_list), ('Seq_len:', self.seqlen_list)]),
+            ('--- Model Computation Configs ---',
+             [('Forward computation time:', getattr(self, 'time_profiled_list', None))]),
+            ('--- Model Memory Configs ---',
+             [('Parameter Memory Cost:', getattr(self, 'param_sizes', None)),
+              ('Activation Memory Cost of Different TP degree (per bsz):',), (getattr(self, 'act_sizes', None),),
+              ('Other Memory Cost (pp = 1):',), (getattr(self, 'other_memory_pp_off', None),),
+              ('Other Memory Cost (pp > 1):',), (getattr(self, 'other_memory_pp_on', None),)]),
+            ('Model Args List:', [(self.model_args_list,)]), ('Train Args List:', [(self.train_args_list,)]),
+            ('Parallel Args List:', [(self.parallel_args_list,)]),
+            ('Profile Model Args List:', [(self.profile_model_args_list,)]),
+            ('Profile Hardware Args List:', [(self.profile_hardware_args_list,)])]
+        for title, lines in sections:
+            print(bar)
+            print(title)
+            for line in lines:
+                print(*line)
+        print(bar)
 
     def get_profiled_model_configs(self):
         args = self.args
@@ -320,6 +370,18 @@ class SearchEngine:
                          layer_num=self.layernum_list, sequence_len=self.seqlen_list, multi_layer_type=True,
                          pp_stage_dict=pp_stage_dict, comm_coe_dict=self.allreduce_comm_coe, gpu_num=args.gpu_num,
                          config=args, **extra)
+
+    def dynamic_programming(self, strategies, bsz, chunk, mbsz_dict, pp_stage_dict, min_tp, max_tp, vsp, embed_sdp,
+                            sp_search, logger=None):
+        """One (task, sp_search) on its own: the ``DpOnModel.fit`` of that task and what the sweep keeps of it
+        (search_engine.py:601-638).  The sweep itself does not go through here: it prepares all tasks first
+        and solves their DP instances together."""
+        model = self._dp_on_model(strategies, pp_stage_dict, logger=logger)
+        check_optimal_chunks(self.args.gpu_num, strategies, self.optimal_chunk_func, bsz, mbsz_dict, min_tp)
+        cost, res_list, pp_deg, remain, mem_cost, vtp = model.fit(bsz, min_tp, max_tp, vsp, embed_sdp, sp_search,
+                                                                  print_=False, mbsz_dict=mbsz_dict)
+        return {'min_cost': cost, 'min_res_list': res_list, 'min_pp_deg': pp_deg, 'mem_remain': remain,
+                'mem_cost': mem_cost, 'throughput': bsz / cost, 'vtp': vtp}
 
     def _spaces(self):
         """(min_tp values, max_tp values, vsp values, embed_sdp values, sp_search values)."""

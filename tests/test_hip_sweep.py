@@ -36,3 +36,25 @@ def test_task_by_task_schedule_gives_the_same(want, tmp_path):
     t = engine.parallelism_optimization(one_batch=False)
     assert S.summarize(engine, t, str(tmp_path))["table"] == want["sweeps"]["two_types_tp"]["table"]
     assert engine.solved_instances > 0 and engine.optimal["bsz"] == 64
+
+
+def test_one_task_on_its_own_gives_its_entry_of_the_sweep(want, tmp_path):
+    """SearchEngine.dynamic_programming -- one (task, sp_search), as the reference's method of that name
+    solves it (search_engine.py:601-638) -- against the same task's entry in the reference's sweep."""
+    engine = S.build(SearchEngine, cost_models, "bsz_range", str(tmp_path))
+    engine.set_searching_bsz()
+    ref = want["sweeps"]["bsz_range"]["table"]
+    seen = 0
+    for task in engine.tasks():
+        bsz, chunk, min_tp, max_tp, vsp, embed_sdp = task
+        for sp_search in engine._spaces()[4]:
+            key = '%d/%d/%d/%d/%d/%d/%d' % (bsz, chunk, min_tp, max_tp, vsp, embed_sdp, sp_search)
+            picked = engine._task_strategies(bsz, chunk, min_tp, max_tp, sp_search)
+            if key not in ref or picked is None:
+                continue
+            cand, mbsz, stage = picked
+            r = engine.dynamic_programming(cand, bsz, chunk, mbsz, stage, min_tp, max_tp, vsp, embed_sdp, sp_search)
+            assert [S.C.hexf(r['throughput']), int(r['min_pp_deg']), S.C.jsonable(r['vtp'])] == ref[key], key
+            assert set(r) == {'min_cost', 'min_res_list', 'min_pp_deg', 'mem_remain', 'mem_cost', 'throughput', 'vtp'}
+            seen += 1
+    assert seen == len(ref)

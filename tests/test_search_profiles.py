@@ -134,3 +134,35 @@ def test_default_locations(tmp_path):
     base = "/m/llama/../../profile_hardware/hardware_configs/"
     assert got == (base + "allreduce_bandwidth_2nodes_4gpus_per_node.json", base + "p2p_bandwidth_2nodes_4gpus_per_node.json",
                    base + "overlap_coefficient.json", base + "sp_time_2nodes_4gpus_per_node.json")
+
+
+def test_search_info_is_printed_on_initialisation(data, tmp_path, capsys):
+    """initialize_search_engine ends with the summary of what the search will work with
+    (search_engine.py:101-106,916-969 of the reference): its section titles and a few of its lines."""
+    engine = P.build(SearchEngine, data, str(tmp_path), P.LOADING_CASES[0])
+    text = capsys.readouterr().out
+    for title in ("--- Optimization Configs ----", "---- Environment Configs ----", "------- Model Configs -------",
+                  "--- Model Computation Configs ---", "--- Model Memory Configs ---", "Model Args List:",
+                  "Profile Hardware Args List:"):
+        assert title in text, title
+    assert "Memory constraint: %d GB" % engine.args.memory_constraint in text
+    assert "Model Name: %s" % engine.model_name in text
+    assert "Layer_num: %s" % engine.layernum_list in text
+
+
+def test_model_type_and_microbatch_function(data, tmp_path):
+    """The two optional setters of the reference's scripts (search_dist.py of every model: set_model_type,
+    set_microbatch_func).  The chunk function they install is called with four arguments everywhere
+    (cost_model.py:79, dynamic_programming.py:224, search_engine.py:1103 of the reference)."""
+    from galvatron_dp.pp_utils import optimal_chunk_func_default
+    engine = P.build(SearchEngine, data, str(tmp_path), P.LOADING_CASES[0])
+    assert engine.model_type == "gpt"
+    engine.set_model_type("bert")
+    assert engine.model_type == "bert"
+    engine.set_microbatch_func(microbatch_size=4, max_chunk=8)
+    strategy = [2, 2, 2, {"fsdp": 0}]
+    for local_bsz, mbsz, min_tp in ((32, 1, 1), (32, 16, 2), (6, 3, 1), (0, 1, 1)):
+        assert engine.optimal_chunk_func(local_bsz, strategy, mbsz, min_tp) == \
+            optimal_chunk_func_default(local_bsz, strategy, 4, min_tp)
+    engine.set_cost_models()
+    assert all(p.optimal_chunk_func is engine.optimal_chunk_func for p in engine.parallel_args_list)
